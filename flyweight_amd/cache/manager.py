@@ -181,6 +181,10 @@ class CacheManager:
             self._native = self._lib.fwh_cache_create(0, windows, default_pages, max_requests, page_size, self.max_pages_per_request)
         if not self._native:
             raise ValueError(host.last_error())
+        for index, (need, _) in enumerate(grouped.values()):
+            kept = int(need.kept_first()) if hasattr(need, "kept_first") else 0
+            if kept and self._lib.fwh_cache_set_keep_first(self._native, index, kept) < 0:
+                raise ValueError(host.last_error())
         for index, (key, (need, entries)) in enumerate(grouped.items()):
             pool = PagePool(borrowed=self._lib.fwh_cache_group_pool(self._native, index), owner=self)
             self.groups.append(PageGroup(key, need, entries, pool, _Tables(self, index)))

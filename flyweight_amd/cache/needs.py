@@ -78,7 +78,8 @@ class PagedKV(CacheNeed):
     keys; a number keeps only the last ``window`` of them, and pages the window has
     passed are given back. ``chunk``: a row sees the keys of its own chunk of that many
     positions only (chunks counted from position 0), and the pages before the chunk of the
-    sequence's next token are given back. K keeps a key's channels together ([page][kv_head][token][channel]:
+    sequence's next token are given back. ``keep_first`` (beside a window): the first so many keys
+    of a sequence stay seen wherever the window stands, and their pages are never given back. K keeps a key's channels together ([page][kv_head][token][channel]:
     the order the scores reduce over), V a channel's tokens ([page][kv_head][channel][token]:
     the order the weighted sum reduces over)."""
 
@@ -87,6 +88,7 @@ class PagedKV(CacheNeed):
     window: Optional[int] = None
     v_head_dim: Optional[int] = None        # the size of a value where it is not the keys' (None: head_dim)
     chunk: Optional[int] = None
+    keep_first: int = 0
     paged = True
 
     def group_key(self) -> Tuple:
@@ -95,7 +97,28 @@ class PagedKV(CacheNeed):
             key += (self.v_head_dim,)
         if self.chunk:
             key += ("chunk", self.chunk)
+        if self.keep_first and self.window:
+            key += ("keep_first", self.keep_first)
         return key
+
+    def kept_first(self) -> int:
+        """Keys at a sequence's start whose pages stay however far a window has moved on."""
+        return int(self.keep_first) if self.window else 0
+
+    def shared_with(self, other: "PagedKV") -> "PagedKV":
+        """The need of a cache entry that a second mixer reads with a mask of its own: the same keys and values,
+        kept for as long as either of the two still sees them."""
+        same = (self.num_kv_heads, self.head_dim, self.v_head_dim or self.head_dim) == \
+            (other.num_kv_heads, other.head_dim, other.v_head_dim or other.head_dim)
+        if not isinstance(other, PagedKV) or not same:
+            raise ValueError(f"cache entries of different shapes cannot be shared: {self} and {other}")
+        if self == other:
+            return self
+        if self.chunk != other.chunk or (self.chunk and (self.window or other.window)):
+            return PagedKV(self.num_kv_heads, self.head_dim, None, self.v_head_dim)      # no common rule: every key is kept
+        window = None if self.window is None or other.window is None else max(self.window, other.window)
+        return PagedKV(self.num_kv_heads, self.head_dim, window, self.v_head_dim, self.chunk,
+                       max(self.keep_first, other.keep_first) if window else 0)
 
     def retention(self) -> int:
         """What the bookkeeping is told: 0 every key is kept, w > 0 the last w, -c < 0 the keys of the next

@@ -3,6 +3,7 @@ from .spec import (ConfigError, LayerSpec, ModelSpec, PartSpec, ScheduleEntry,
 from .lfm2 import Lfm2Config
 from .koketar import KoketarConfig
 from .vavelorn import VavelornConfig
+from .dalerax import DaleraxConfig
 from .registry import (architecture_name, config_from_dict, load_config,
                        register_architecture, registered_architectures)
 
@@ -10,9 +11,10 @@ register_architecture("Lfm2ForCausalLM", Lfm2Config)
 register_architecture("lfm2", Lfm2Config)
 register_architecture("Koketar", KoketarConfig)
 register_architecture("Vavelorn", VavelornConfig)
+register_architecture("Dalerax", DaleraxConfig)
 
 __all__ = [
     "ConfigError", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry", "default_schedule",
-    "Lfm2Config", "KoketarConfig", "VavelornConfig", "architecture_name", "config_from_dict", "load_config",
+    "Lfm2Config", "KoketarConfig", "VavelornConfig", "DaleraxConfig", "architecture_name", "config_from_dict", "load_config",
     "register_architecture", "registered_architectures",
 ]

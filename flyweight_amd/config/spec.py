@@ -88,6 +88,8 @@ class ModelSpec:
     embedding_scale: float = 1.0
     logit_scale: float = 1.0
     logit_softcap: float = 0.0
+    # a table [max_positions, hidden] of learned vectors, one per position, added to the embedding rows (None: none)
+    position_table_name: Optional[str] = None
 
     def validate(self) -> None:
         if self.hidden_size <= 0 or self.vocab_size <= 0:

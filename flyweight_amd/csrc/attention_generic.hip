@@ -22,12 +22,11 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, int interleaved) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, int interleaved, int width) {
     __shared__ float normed[ATTN_MAX_HEAD_DIM];
     const int row = blockIdx.x;
     const int vec = blockIdx.y;
     const int lane = threadIdx.x;
-    const int width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
     const TI* source = qkv + (size_t)row * width + (vec < num_heads + num_kv_heads
                            ? (size_t)vec * head_dim
                            : (size_t)(num_heads + num_kv_heads) * head_dim + (size_t)(vec - num_heads - num_kv_heads) * v_dim);
@@ -90,11 +89,10 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows, int interleaved) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows, int interleaved, int width) {
     const int r0 = blockIdx.x * QK_ROWS;
     const int vec = blockIdx.y;
     const int lane = threadIdx.x;
-    const int width = (num_heads + 2 * num_kv_heads) * head_dim;
     const bool active = lane < head_dim;
     const bool is_value = vec >= num_heads + num_kv_heads, is_query = vec < num_heads;
     const float* weight = is_value ? nullptr : (is_query ? q_norm_weight : k_norm_weight);
@@ -172,7 +170,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
                                         const int32_t* block_table, int table_stride, const int32_t* row_seg,
                                         const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                                         int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved,
-                                        void* stream) {
+                                        int q_only, void* stream) {
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0, "qk_norm_rope: bad sizes rows=%d heads=%d kv_heads=%d", rows, num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
@@ -183,7 +181,9 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
     FW_REQUIRE((q_norm_weight == nullptr) == (k_norm_weight == nullptr), "qk_norm_rope: q and k norm weights come together");
     FW_REQUIRE(rows <= 1 << 20, "qk_norm_rope: too many rows (%d)", rows);
     if (rows == 0) return 0;
+    FW_REQUIRE(!(q_only && write_kv), "qk_norm_rope: rows that hold queries only bring no keys or values to store");
     const int vectors = write_kv ? num_heads + 2 * num_kv_heads : num_heads;
+    const int width = q_only ? num_heads * head_dim : (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
     FW_REQUIRE(vectors <= 65535, "qk_norm_rope: too many heads (%d)", vectors);
     dim3 grid(rows, vectors);
     hipStream_t s = (hipStream_t)stream;
@@ -192,7 +192,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_ROWS_LAUNCH(TI, T)                                                                                     \
     qk_norm_rope_kv_write_rows_kernel<TI, T><<<by_rows, 64, 0, s>>>(                                                 \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows, interleaved)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows, interleaved, width)
         if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_ROWS_LAUNCH(float, float);
         else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(float, bf16_t);
         else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(bf16_t, bf16_t);
@@ -204,7 +204,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_LAUNCH(TI, T)                                                                                          \
     qk_norm_rope_kv_write_kernel<TI, T><<<grid, 64, 0, s>>>(                                                         \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, interleaved)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, interleaved, width)
     if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_LAUNCH(float, float);
     else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_LAUNCH(float, bf16_t);
     else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_LAUNCH(bf16_t, bf16_t);
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
     const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
-    int chunk, float softcap) {
+    int chunk, float softcap, int keep_first, const float* __restrict__ sinks) {
     __shared__ float qs[ATTN_MAX_HEAD_DIM];
     __shared__ float ps[ATTN_PAGE];
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -237,10 +237,15 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const int first = fw_first_visible(pos, window, chunk);
     float running_max = -INFINITY, running_sum = 0.0f;
     float acc[ATTN_MAX_HEAD_DIM / 64] = {};
-    for (int tile = first / ATTN_PAGE; tile <= pos / ATTN_PAGE; ++tile) {
+    // the pages of the kept first keys that lie before the first visible one, then those from it on
+    const int kept = keep_first < first ? keep_first : first;              // keys 0 .. kept - 1 are seen beside first .. pos
+    const int head_tiles = (kept + ATTN_PAGE - 1) / ATTN_PAGE < first / ATTN_PAGE ? (kept + ATTN_PAGE - 1) / ATTN_PAGE : first / ATTN_PAGE;
+    const int tiles = head_tiles + pos / ATTN_PAGE - first / ATTN_PAGE + 1;
+    for (int at = 0; at < tiles; ++at) {
+        const int tile = at < head_tiles ? at : first / ATTN_PAGE + at - head_tiles;
         const int page = table[tile];
         const int t = tile * ATTN_PAGE + lane;
-        const bool valid = t >= first && t <= pos;
+        const bool valid = (t >= first || t < kept) && t <= pos;
         float score = -INFINITY;
         if (valid) {
             const T* key = k_pages + (((size_t)page * num_kv_heads + kvh) * ATTN_PAGE + lane) * head_dim;
@@ -256,7 +261,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         running_max = new_max;
         ps[lane] = p;
         __syncthreads();
-        const int lo = first - tile * ATTN_PAGE > 0 ? first - tile * ATTN_PAGE : 0;
+        const int lo = (first - tile * ATTN_PAGE > 0 && kept <= tile * ATTN_PAGE) ? first - tile * ATTN_PAGE : 0;    // a masked key's weight is 0
         const int hi = pos - tile * ATTN_PAGE < ATTN_PAGE - 1 ? pos - tile * ATTN_PAGE : ATTN_PAGE - 1;
 #pragma unroll
         for (int j = 0; j < ATTN_MAX_HEAD_DIM / 64; ++j) {
@@ -270,11 +275,18 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
         }
         __syncthreads();
     }
+    float shrink = 1.0f;
+    if (sinks) {        // one more term in the sum, with no value: exp(sink), not scaled
+        const float sink = sinks[head];
+        const float new_max = fmaxf(running_max, sink);
+        shrink = expf(running_max - new_max);
+        running_sum = running_sum * shrink + expf(sink - new_max);
+    }
     T* dest = out + ((size_t)row * num_heads + head) * v_dim;
 #pragma unroll
     for (int j = 0; j < ATTN_MAX_HEAD_DIM / 64; ++j) {
         const int d = lane + 64 * j;
-        if (d < v_dim) store_from_float(dest, d, acc[j] / running_sum);
+        if (d < v_dim) store_from_float(dest, d, acc[j] * shrink / running_sum);
     }
 }
 
@@ -282,8 +294,9 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
                                     const void* v_pages, const int32_t* block_table, int table_stride,
                                     const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                     int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk,
-                                    float softcap, int page_size, int num_pages, void* stream) {
+                                    float softcap, int keep_first, const float* sinks, int page_size, int num_pages, void* stream) {
     FW_REQUIRE(chunk >= 0 && softcap >= 0.0f, "attention: chunk %d and soft cap %g must not be negative", chunk, (double)softcap);
+    FW_REQUIRE(keep_first >= 0 && (keep_first == 0 || chunk == 0), "attention: %d first keys are kept beside a window, not beside chunks", keep_first);
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
                "attention: heads %d must be a positive multiple of kv heads %d", num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "attention: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
@@ -297,11 +310,11 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
     if (dtype == FW_F32)
         attention_generic_kernel<float><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, keep_first, sinks);
     else if (dtype == FW_BF16)
         attention_generic_kernel<bf16_t><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, keep_first, sinks);
     else
         FW_REQUIRE(false, "attention: unknown dtype %d", dtype);
     FW_LAUNCH_CHECK("attention_generic");

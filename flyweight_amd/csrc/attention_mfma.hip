@@ -56,7 +56,7 @@ struct Columns {
 // One page of 64 keys against NH sets of columns that share the keys (query heads of one kv
 // group over the same rows): the keys and values are read once for all of them. `lo`/`hi`: the
 // keys of this page that this lane's column may see are those with lo <= key <= hi
-// (page-relative; hi < 0: none). `last_written`: keys beyond it hold whatever an earlier owner of
+// (page-relative; hi < 0: none), and with `kept` > 0 also the keys below `kept`. `last_written`: keys beyond it hold whatever an earlier owner of
 // the page left, and are zeroed before they meet P = 0: here if CLEAN_V, else the caller has done
 // it (the prompt kernel does when it copies a page to LDS). K_PADDED: a key's row holds HD channels,
 // those past head_dim zero (the prompt kernel's LDS tile), so every lane loads; else the lanes past
@@ -75,7 +75,7 @@ template <int HD, int NH, bool CLEAN_V, bool K_PADDED, bool EARLY_V = false>
 __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
                                             const uint16_t* __restrict__ v_page, int head_dim, int v_dim, float scale_log2,
                                             int lo, int hi, int last_written, int k_stride, int v_stride,
-                                            float cap = 0.0f, float cap_scale = 0.0f) {
+                                            float cap = 0.0f, float cap_scale = 0.0f, int kept = 0) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
     // all key loads of the page are issued before the first product
@@ -133,14 +133,15 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
                     s[h][kt][r] = cap - 2.0f * cap * __builtin_amdgcn_rcpf(1.0f + e);
                 }
     }
-    const bool full = __all(lo <= 0 && hi >= PAGE - 1) && last_written >= PAGE - 1;
+    // `kept`: the keys below it (page-relative; <= 0: none) are seen as well, whatever `lo` says
+    const bool full = __all((lo <= 0 || kept >= lo) && hi >= PAGE - 1) && last_written >= PAGE - 1;
     if (!full) {
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = kt * 16 + g * 4 + r;
-                const bool seen = key >= lo && key <= hi;
+                const bool seen = (key >= lo || key < kept) && key <= hi;
 #pragma unroll
                 for (int h = 0; h < NH; ++h) s[h][kt][r] = seen ? s[h][kt][r] : NEG_BIG;
             }
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
     const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale_log2, int window,
-    int chunk, float cap, float cap_scale) {
+    int chunk, float cap, float cap_scale, int keep_first, const float* __restrict__ sinks) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     // a key's row in LDS holds HD channels, those past head_dim zero: every lane loads its operand
     constexpr int k_stride = HD + KV_PAD;
@@ -332,7 +333,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     // flight while the page before them is worked on.
     const int k_runs = PAGE * head_dim / 8, v_runs = PAGE * v_dim / 8;
     constexpr int MAX_RUNS = HD * PAGE / 8 / 256;                                // per thread, per operand
-    const int first_block = tile_first / PAGE, last_block = pos_hi / PAGE;
+    // The pages a tile walks: those of the kept first keys that lie before the window's first page, then
+    // the window's. `step` numbers them; block_of gives the page's place in the sequence.
+    const int window_block = tile_first / PAGE, last_block = pos_hi / PAGE;
+    const int kept_blocks = (keep_first + PAGE - 1) / PAGE < window_block ? (keep_first + PAGE - 1) / PAGE : window_block;
+    const int last_step = kept_blocks + last_block - window_block;
+    auto block_of = [&](int step) { return step < kept_blocks ? step : window_block + step - kept_blocks; };
     u32x4 hold_k0[MAX_RUNS], hold_v0[MAX_RUNS], hold_k1[MAX_RUNS], hold_v1[MAX_RUNS];
     // what a thread copies of every page: fixed offsets, so that a page's address is a scalar
     // base plus these (no vector arithmetic per page; the registers that receive a page are
@@ -343,8 +349,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
         run_offset[u] = (uint32_t)(tid + u * 256 < k_runs ? tid + u * 256 : 0) * 8u;
         run_offset_v[u] = (uint32_t)(tid + u * 256 < v_runs ? tid + u * 256 : 0) * 8u;
     }
-    auto fetch = [&](u32x4 (&hold_k)[MAX_RUNS], u32x4 (&hold_v)[MAX_RUNS], int block) {
-        const int page = __builtin_amdgcn_readfirstlane(table[block < last_block ? block : last_block]);
+    auto fetch = [&](u32x4 (&hold_k)[MAX_RUNS], u32x4 (&hold_v)[MAX_RUNS], int step) {
+        const int page = __builtin_amdgcn_readfirstlane(table[block_of(step < last_step ? step : last_step)]);
         const uint16_t* k_from = k_pages + ((size_t)page * num_kv_heads + kvh) * k_page_elems;
         const uint16_t* v_from = v_pages + ((size_t)page * num_kv_heads + kvh) * v_page_elems;
 #pragma unroll
@@ -355,7 +361,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     };
     // The values of keys past the last one written (only in the tile's last page) are zeroed on
     // their way to LDS: whatever an earlier owner of the page left there must not meet P = 0.
-    auto stash = [&](const u32x4 (&hold_k)[MAX_RUNS], const u32x4 (&hold_v)[MAX_RUNS], int buffer, int block) {
+    auto stash = [&](const u32x4 (&hold_k)[MAX_RUNS], const u32x4 (&hold_v)[MAX_RUNS], int buffer, int step) {
+        const int block = block_of(step);
         uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
         uint16_t* vt = kt + k_elems;
         const int k_per_row = head_dim / 8;
@@ -378,41 +385,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
             }
         }
     };
-    auto attend = [&](int block, int buffer) {
-        const int base = block * PAGE;
+    auto attend = [&](int step, int buffer) {
+        const int base = block_of(step) * PAGE;
         if (rows > 0 && base <= wave_hi) {      // a wave whose rows all lie before this page has nothing to add
             const uint16_t* kt = lds + (size_t)buffer * (k_elems + v_elems);
             // a lane without a row computes along with the bounds of the tile's first row (nothing of
             // it is stored): a page that is whole for the rows is then whole for the wave
             attend_page<HD, NH, false, true>(c, kt, kt + k_elems, head_dim, v_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
-                            k_stride, v_stride, cap, cap_scale);
+                            k_stride, v_stride, cap, cap_scale, keep_first - base);
         }
     };
 
     // page b travels: global -> register set (b - first) % 2, requested two pages ahead -> LDS
     // buffer (b - first) % 2, stored while page b - 1 is worked on -> attended
-    fetch(hold_k0, hold_v0, first_block);
-    fetch(hold_k1, hold_v1, first_block + 1);
-    stash(hold_k0, hold_v0, 0, first_block);
+    fetch(hold_k0, hold_v0, 0);
+    fetch(hold_k1, hold_v1, 1);
+    stash(hold_k0, hold_v0, 0, 0);
     fw_lds_barrier();
-    for (int block = first_block; block <= last_block; block += 2) {
-        fetch(hold_k0, hold_v0, block + 2);
+    for (int step = 0; step <= last_step; step += 2) {
+        fetch(hold_k0, hold_v0, step + 2);
         __builtin_amdgcn_sched_barrier(0);      // keep the requests ahead of the work they overlap
-        attend(block, 0);
-        stash(hold_k1, hold_v1, 1, block + 1);
+        attend(step, 0);
+        stash(hold_k1, hold_v1, 1, step + 1);
         fw_lds_barrier();
-        if (block + 1 > last_block) break;
-        fetch(hold_k1, hold_v1, block + 3);
+        if (step + 1 > last_step) break;
+        fetch(hold_k1, hold_v1, step + 3);
         __builtin_amdgcn_sched_barrier(0);
-        attend(block + 1, 1);
-        stash(hold_k0, hold_v0, 0, block + 2);
+        attend(step + 1, 1);
+        stash(hold_k0, hold_v0, 0, step + 2);
         fw_lds_barrier();
     }
 #pragma unroll
     for (int h = 0; h < NH; ++h) {
-        const float l = fw_quad_sum(c[h].l);
+        float l = fw_quad_sum(c[h].l);
         if (!valid || first_in_group + h >= group) continue;
-        const float inv = 1.0f / l;
+        float inv = 1.0f / l;
+        if (sinks) {        // one more term in the sum, with no value: exp(sink), not scaled
+            const float sink = sinks[kvh * group + first_in_group + h] * 1.4426950408889634f;
+            const float top = fmaxf(c[h].m, sink);
+            const float shrink = exp2f(c[h].m - top);
+            inv = shrink / (l * shrink + exp2f(sink - top));
+        }
         uint16_t* dest = out + ((size_t)my_row * num_heads + kvh * group + first_in_group + h) * v_dim;
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t) {
@@ -449,6 +462,7 @@ struct FusedProjections {
     int rotary_dim;
     int write_kv;                   // 0: another execution of the layer has stored this step's keys and values already
     int interleaved;                // 0: channel i turns with channel i + rotary_dim / 2; 1: channel 2i with channel 2i + 1
+    int width;                      // floats of a row of qkv: queries alone where the keys and values are another layer's
 };
 
 // One head-vector of head_dim channels by one wave: optional RMS norm, then the half-split rotation
@@ -496,7 +510,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     uint16_t* k_pages, uint16_t* v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
     int head_dim, int v_dim, float scale_log2, int window, int chunk, float cap, float cap_scale, int max_splits,
-    const int32_t* __restrict__ decode_work, const FusedProjections fused) {
+    const int32_t* __restrict__ decode_work, const FusedProjections fused, int keep_first, const float* __restrict__ sinks) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
@@ -524,9 +538,13 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         rounds = rounds < 1 ? 1 : rounds;
     }
     const int pages_per_split = SPLIT_PAGES * rounds;
-    const int first_block = first / PAGE + split * pages_per_split;
-    const int last_block = pos / PAGE;
-    if (first_block > last_block) return;       // the whole workgroup
+    // The pages a row walks: those of the kept first keys that lie before the window's first page, then the
+    // window's. They are numbered through (`step`), and the splits are counted over the steps.
+    const int window_block = first / PAGE, last_block = pos / PAGE;
+    const int kept_blocks = (keep_first + PAGE - 1) / PAGE < window_block ? (keep_first + PAGE - 1) / PAGE : window_block;
+    const int last_step = kept_blocks + last_block - window_block;
+    const int first_step = split * pages_per_split;
+    if (first_step > last_step) return;         // the whole workgroup
     const int in_group = head_tile * 16 + col;
     const bool valid = in_group < group;
     const int head = kvh * group + (valid ? in_group : 0);
@@ -534,15 +552,14 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     Columns<HD> columns_of_wave[1];
     Columns<HD>& c = columns_of_wave[0];
     if (FUSED) {
-        const int width = (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
-        const float* projections = fused.qkv + (size_t)row * width;
+        const float* projections = fused.qkv + (size_t)row * fused.width;
         const int half = fused.rotary_dim / 2;
         const float* cos_row = fused.cos_table + (size_t)row * half;
         const float* sin_row = fused.sin_table + (size_t)row * half;
         const int columns = group - head_tile * 16 < 16 ? group - head_tile * 16 : 16;
         // the vectors of this workgroup: its query heads, then (where the row's own position lies
         // in its pages) the new key and the new value; a wave takes every fourth
-        const bool stores = fused.write_kv && last_block < first_block + pages_per_split;
+        const bool stores = fused.write_kv && last_step < first_step + pages_per_split;
         const int vectors = columns + (stores ? 2 : 0);
         const int slot = pos % PAGE;
         const int own_page = stores ? block_table[(size_t)segment * table_stride + last_block] : 0;
@@ -571,14 +588,15 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
     }
     for (int round = 0; round < rounds; ++round) {
-        const int block = first_block + round * SPLIT_PAGES + wave;
-        if (block > last_block) break;
+        const int step = first_step + round * SPLIT_PAGES + wave;
+        if (step > last_step) break;
+        const int block = step < kept_blocks ? step : window_block + step - kept_blocks;
         const int page = block_table[(size_t)segment * table_stride + block];
         const size_t at = ((size_t)page * num_kv_heads + kvh) * PAGE;
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
         attend_page<HD, 1, true, false, (HD <= 128)>(columns_of_wave, k_pages + at * head_dim, v_pages + at * v_dim, head_dim, v_dim, scale_log2, first - base, pos - base, pos - base,
-                        head_dim, PAGE, cap, cap_scale);
+                        head_dim, PAGE, cap, cap_scale, keep_first - base);
     }
     const float l = fw_quad_sum(c.l);
 #pragma unroll
@@ -589,13 +607,18 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     }
     __syncthreads();
     // how many workgroups work on this row: those whose first page holds a visible key
-    const int row_splits = (last_block - first / PAGE + 1 + pages_per_split - 1) / pages_per_split;
+    const int row_splits = (last_step + 1 + pages_per_split - 1) / pages_per_split;
+    // the sink of a head: one more part of the row, with maximum sink, sum 1 and no output (in units of log2)
+    const float LOG2E_F = 1.4426950408889634f;
     const int stride = PART_STRIDE(v_dim);
     if (valid) {        // every wave: the four share out the channel tiles, each storing a quarter of the workgroup's result
         float m = NEG_BIG;
 #pragma unroll
         for (int w = 0; w < SPLIT_PAGES; ++w) m = fmaxf(m, shared_m[w][col]);
-        float total = 0.0f, weight[SPLIT_PAGES];
+        const bool final_here = row_splits == 1;
+        const float sink = (sinks && final_here) ? sinks[head] * LOG2E_F : NEG_BIG;
+        m = fmaxf(m, sink);
+        float total = (sinks && final_here) ? exp2f(sink - m) : 0.0f, weight[SPLIT_PAGES];
 #pragma unroll
         for (int w = 0; w < SPLIT_PAGES; ++w) {
             weight[w] = exp2f(shared_m[w][col] - m);        // a wave without a page has l = 0 and o = 0
@@ -667,6 +690,11 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
                     }
             }
             float total = 0.0f;
+            if (sinks) {
+                const float sink = sinks[kvh * group + head_tile * 16 + threadIdx.x] * LOG2E_F;
+                m = fmaxf(m, sink);
+                total = exp2f(sink - m);
+            }
             for (int sp = 0; sp < row_splits; ++sp) {
                 const float weight = exp2f(merge_w[sp][threadIdx.x] - m);
                 total += weight * merge_l[sp][threadIdx.x];
@@ -725,6 +753,10 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         };
         constexpr int AT_ONCE = 16;
         float m = NEG_BIG, total = 0.0f, acc = 0.0f;
+        if (sinks) {
+            m = sinks[merged_head] * LOG2E_F;
+            total = 1.0f;
+        }
         for (int sp0 = 0; sp0 < row_splits; sp0 += AT_ONCE) {
             float ms[AT_ONCE], ls[AT_ONCE], vs[AT_ONCE];
 #pragma unroll
@@ -802,8 +834,9 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
                                     const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                                     const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
                                     const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim,
-                                    int v_dim, float scale, int window, int chunk, float softcap, int page_size, int num_pages,
-                                    int heads_together, void* stream) {
+                                    int v_dim, float scale, int window, int chunk, float softcap, int keep_first, const float* sinks,
+                                    int page_size, int num_pages, int heads_together, void* stream) {
+    FW_REQUIRE(keep_first >= 0 && (keep_first == 0 || chunk == 0), "attention_prefill: %d first keys are kept beside a window, not beside chunks", keep_first);
     if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride, chunk, softcap)) return -1;
     const ScoreRule rule = score_rule(scale, softcap);
     const int widest = head_dim > v_dim ? head_dim : v_dim;      // the template holds both
@@ -831,7 +864,7 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
         attention_prefill_kernel<HD, NH><<<grid, 256, lds_bytes, (hipStream_t)stream>>>(                            \
             (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,    \
             table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, v_dim,        \
-            rule.scale_log2, window, chunk, rule.cap, rule.cap_scale);                                             \
+            rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, keep_first, sinks);                          \
     }
     if (widest <= 32) {
         if (heads_together == 4) LAUNCH(32, 4) else LAUNCH(32, 1)
@@ -848,13 +881,16 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
 }
 
 static int decode_check(int max_splits, int max_context, int* tickets, int tickets_len, int table_stride, int rows, int num_heads,
-                        int num_kv_heads, int head_dim, int v_dim, int window, int page_size, int num_pages, int chunk, float softcap) {
+                        int num_kv_heads, int head_dim, int v_dim, int window, int page_size, int num_pages, int chunk, float softcap,
+                        int keep_first = 0) {
+    FW_REQUIRE(keep_first >= 0 && (keep_first == 0 || chunk == 0), "attention_decode: %d first keys are kept beside a window, not beside chunks", keep_first);
     if (check_common("attention_decode", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride, chunk, softcap)) return -1;
     window = visible_span(window, chunk);       // below: what bounds the pages a row's keys lie in
     FW_REQUIRE(max_splits >= 1 && max_splits <= 65535, "attention_decode: max_splits %d outside 1..65535", max_splits);
     FW_REQUIRE(max_context >= 1, "attention_decode: max_context must be positive");
     int blocks = (max_context + PAGE - 1) / PAGE;
-    if (window > 0 && (window + PAGE - 2) / PAGE + 1 < blocks) blocks = (window + PAGE - 2) / PAGE + 1;
+    if (window > 0 && (window + PAGE - 2) / PAGE + 1 + (keep_first + PAGE - 1) / PAGE < blocks)
+        blocks = (window + PAGE - 2) / PAGE + 1 + (keep_first + PAGE - 1) / PAGE;
     FW_REQUIRE(max_splits * SPLIT_PAGES >= blocks, "attention_decode: %d splits of %d pages do not cover %d pages of context",
                max_splits, SPLIT_PAGES, blocks);
     FW_REQUIRE((max_context + PAGE - 1) / PAGE <= table_stride, "attention_decode: a context of %d tokens exceeds the block table (%d pages)",
@@ -869,7 +905,7 @@ static int decode_check(int max_splits, int max_context, int* tickets, int ticke
 static int decode_launch(const void* q, void* out, float* partial, int max_splits, const int32_t* decode_work, int* tickets, void* k_pages, void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* row_seg, const int32_t* row_pos, int rows,
                          int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                         const FusedProjections& fused, void* stream) {
+                         const FusedProjections& fused, int keep_first, const float* sinks, void* stream) {
     if (rows == 0) return 0;
     const ScoreRule rule = score_rule(scale, softcap);
     const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
@@ -879,11 +915,11 @@ static int decode_launch(const void* q, void* out, float* partial, int max_split
     if (fused.qkv)                                                                                                            \
         attention_decode_split_kernel<HD, true><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                          \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused); \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused, keep_first, sinks); \
     else                                                                                                                      \
         attention_decode_split_kernel<HD, false><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                         \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused)
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused, keep_first, sinks)
     FW_BY_HEAD_DIM((head_dim > v_dim ? head_dim : v_dim), CALL);
 #undef CALL
     FW_LAUNCH_CHECK("attention_decode");
@@ -903,11 +939,11 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
                                    const void* v_pages, const int32_t* block_table, int table_stride,
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                    int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                                   int page_size, int num_pages, void* stream) {
+                                   int keep_first, const float* sinks, int page_size, int num_pages, void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
-                     page_size, num_pages, chunk, softcap)) return -1;
+                     page_size, num_pages, chunk, softcap, keep_first)) return -1;
     return decode_launch(q, out, partial, max_splits, decode_work, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
-                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, FusedProjections{}, stream);
+                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, FusedProjections{}, keep_first, sinks, stream);
 }
 
 // fw_attention_decode with the work of fw_qk_norm_rope_kv_write in front of it, in the same kernel:
@@ -921,9 +957,11 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
                                          void* k_pages, void* v_pages, const int32_t* block_table, int table_stride,
                                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                          int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                                         int interleaved, int page_size, int num_pages, void* stream) {
+                                         int interleaved, int q_only, int keep_first, const float* sinks, int page_size, int num_pages,
+                                         void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
-                     page_size, num_pages, chunk, softcap)) return -1;
+                     page_size, num_pages, chunk, softcap, keep_first)) return -1;
+    FW_REQUIRE(!(q_only && write_kv), "attention_decode_fused: rows that hold queries only bring no keys or values to store");
     FW_REQUIRE(qkv != nullptr, "attention_decode_fused: the projections are missing");
     FW_REQUIRE(rotary_dim >= 0 && rotary_dim <= head_dim && rotary_dim % 2 == 0, "attention_decode_fused: rotary_dim %d with head_dim %d",
                rotary_dim, head_dim);
@@ -933,6 +971,7 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
     fused.qkv = qkv; fused.q_norm_weight = q_norm_weight; fused.k_norm_weight = k_norm_weight; fused.eps = eps;
     fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rotary_dim = rotary_dim; fused.write_kv = write_kv;
     fused.interleaved = interleaved;
+    fused.width = q_only ? num_heads * head_dim : (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
     return decode_launch(nullptr, out, partial, max_splits, decode_work, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
-                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, fused, stream);
+                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, fused, keep_first, sinks, stream);
 }

@@ -358,13 +358,14 @@ extern "C" int fw_gated_delta_rule(const float* records, float* state, float* ou
 template <typename TG, typename T>
 __global__ __launch_bounds__(64) void gated_head_norm_kernel(const float* __restrict__ o, const TG* __restrict__ gate, int gate_stride,
                                                             const float* __restrict__ weight, T* __restrict__ out,
-                                                            int heads, int vdim, float eps, int gate_silu) {
+                                                            int heads, int vdim, float eps, int gate_silu, int weight_per_head) {
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
     const float* source = o + ((size_t)row * heads + head) * vdim;
     float sum = 0.0f;
     for (int j = lane; j < vdim; j += 64) sum += source[j] * source[j];
     sum = wave_sum(sum);
     const float inv = 1.0f / sqrtf(sum / (float)vdim + eps);
+    if (weight_per_head) weight += (size_t)head * vdim;       // every head has a weight of its own, [heads][vdim]
     for (int j = lane; j < vdim; j += 64) {
         const float z = load_as_float(gate, (size_t)row * gate_stride + head * vdim + j);
         const float g = gate_silu ? z * fw_sigmoid(z) : fw_sigmoid(z);
@@ -373,14 +374,14 @@ __global__ __launch_bounds__(64) void gated_head_norm_kernel(const float* __rest
 }
 
 extern "C" int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight,
-                                  void* out, int out_dtype, int rows, int heads, int vdim, float eps, int gate_silu, void* stream) {
+                                  int weight_per_head, void* out, int out_dtype, int rows, int heads, int vdim, float eps, int gate_silu, void* stream) {
     FW_REQUIRE(rows >= 0 && heads > 0 && heads <= 65535 && vdim > 0, "gated_head_norm: bad sizes rows=%d heads=%d vdim=%d", rows, heads, vdim);
     FW_REQUIRE(gate_stride >= heads * vdim, "gated_head_norm: the gates' rows (%d wide) do not hold %d x %d", gate_stride, heads, vdim);
     if (rows == 0) return 0;
     dim3 grid(rows, heads);
     hipStream_t s = (hipStream_t)stream;
 #define FW_GHN_LAUNCH(TG, T) \
-    gated_head_norm_kernel<TG, T><<<grid, 64, 0, s>>>(o, (const TG*)gate, gate_stride, weight, (T*)out, heads, vdim, eps, gate_silu)
+    gated_head_norm_kernel<TG, T><<<grid, 64, 0, s>>>(o, (const TG*)gate, gate_stride, weight, (T*)out, heads, vdim, eps, gate_silu, weight_per_head)
     if (gate_dtype == FW_F32 && out_dtype == FW_F32) FW_GHN_LAUNCH(float, float);
     else if (gate_dtype == FW_F32 && out_dtype == FW_BF16) FW_GHN_LAUNCH(float, bf16_t);
     else if (gate_dtype == FW_BF16 && out_dtype == FW_BF16) FW_GHN_LAUNCH(bf16_t, bf16_t);

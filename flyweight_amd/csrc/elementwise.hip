@@ -16,33 +16,44 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 14; }
+extern "C" int fw_abi_version(void) { return 15; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
 // (native/include/flyweight_v2_native_kernels.hpp:98-151).
 // `scale` multiplies the row (architectures that scale their embeddings; 1 leaves it as stored).
-template <typename W>
+template <typename W, typename P>
 __global__ void embed_rows_kernel(const W* __restrict__ table, const int32_t* __restrict__ ids,
-                                  float* __restrict__ out, int hidden, float scale) {
+                                  float* __restrict__ out, int hidden, float scale, const P* __restrict__ places_table,
+                                  const int32_t* __restrict__ places) {
     const int row = blockIdx.y;
     const size_t base = (size_t)ids[row] * hidden;
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < hidden; i += gridDim.x * blockDim.x)
-        out[(size_t)row * hidden + i] = load_as_float(table, base + i) * scale;
+    const size_t place = places ? (size_t)places[row] * hidden : 0;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < hidden; i += gridDim.x * blockDim.x) {
+        float value = load_as_float(table, base + i) * scale;
+        if (places) value += load_as_float(places_table, place + i);
+        out[(size_t)row * hidden + i] = value;
+    }
 }
 
 extern "C" int fw_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out,
-                             int rows, int hidden, int vocab, float scale, void* stream) {
+                             int rows, int hidden, int vocab, float scale, const void* places_table, int places_dtype,
+                             const int32_t* places, int places_entries, void* stream) {
     FW_REQUIRE(rows >= 0 && hidden > 0 && vocab > 0, "embed_rows: bad sizes rows=%d hidden=%d vocab=%d", rows, hidden, vocab);
     FW_REQUIRE(rows <= 65535, "embed_rows: at most 65535 rows per call, got %d", rows);
+    FW_REQUIRE(places == nullptr || (places_table != nullptr && places_entries > 0), "embed_rows: places without a table of them");
     if (rows == 0) return 0;
     dim3 grid(fw_ceil_div(hidden, 256) > 64 ? 64 : fw_ceil_div(hidden, 256), rows);
-    if (table_dtype == FW_F32)
-        embed_rows_kernel<float><<<grid, 256, 0, (hipStream_t)stream>>>((const float*)table, ids, out, hidden, scale);
-    else if (table_dtype == FW_BF16)
-        embed_rows_kernel<bf16_t><<<grid, 256, 0, (hipStream_t)stream>>>((const bf16_t*)table, ids, out, hidden, scale);
-    else
-        FW_REQUIRE(false, "embed_rows: unknown table dtype %d", table_dtype);
+    hipStream_t s = (hipStream_t)stream;
+    if (places == nullptr) places_dtype = table_dtype;
+#define FW_EMBED_LAUNCH(W, P) \
+    embed_rows_kernel<W, P><<<grid, 256, 0, s>>>((const W*)table, ids, out, hidden, scale, (const P*)places_table, places)
+    if (table_dtype == FW_F32 && places_dtype == FW_F32) FW_EMBED_LAUNCH(float, float);
+    else if (table_dtype == FW_BF16 && places_dtype == FW_BF16) FW_EMBED_LAUNCH(bf16_t, bf16_t);
+    else if (table_dtype == FW_BF16 && places_dtype == FW_F32) FW_EMBED_LAUNCH(bf16_t, float);
+    else if (table_dtype == FW_F32 && places_dtype == FW_BF16) FW_EMBED_LAUNCH(float, bf16_t);
+    else FW_REQUIRE(false, "embed_rows: unknown table dtypes %d, %d", table_dtype, places_dtype);
+#undef FW_EMBED_LAUNCH
     FW_LAUNCH_CHECK("embed_rows");
     return 0;
 }

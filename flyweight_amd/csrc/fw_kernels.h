@@ -14,9 +14,11 @@ extern "C" {
 const char* fw_last_error(void);
 int fw_abi_version(void);
 
-// out[r][:] = table[ids[r]][:] * scale  (float32 out: the residual stream)
+// out[r][:] = table[ids[r]][:] * scale  (float32 out: the residual stream); with a second table (places
+// null: none) + places_table[places[r]][:], not scaled (a learned vector per position)
 int fw_embed_rows(const void* table, int table_dtype, const int32_t* ids, float* out,
-                  int rows, int hidden, int vocab, float scale, void* stream);
+                  int rows, int hidden, int vocab, float scale, const void* places_table, int places_dtype,
+                  const int32_t* places, int places_entries, void* stream);
 
 // x <- x * scale, then with cap > 0: x <- cap * tanh(x / cap); float32, in place
 int fw_scale_softcap(float* x, long long count, float scale, float cap, void* stream);
@@ -131,16 +133,20 @@ int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dty
                              const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                              const int32_t* block_table, int table_stride, const int32_t* row_seg,
                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved, void* stream);
+                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved, int q_only, void* stream);
 
 // Causal attention of every row over the cached keys 0..row_pos[r] of its segment, or the last `window`
 // of them, or with `chunk` > 0 those of its own chunk of that many positions (counted from position 0
 // of the sequence); softcap c > 0: score <- c * tanh(score / c) after the scale. out [rows][nh*vd].
+// keep_first n > 0 (beside a window): the first n keys of the sequence are seen as well, wherever the window
+// stands. sinks (float32 [heads], or null): one more term exp(sinks[head]) in the softmax's denominator, with
+// no key and no value, not scaled. (q_only of fw_qk_norm_rope_kv_write / fw_attention_decode_fused: the rows
+// of qkv hold the queries alone, [heads * head_dim]: the keys and values are another layer's.)
 int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                          const void* v_pages, const int32_t* block_table, int table_stride,
                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                          int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                         int page_size, int num_pages, void* stream);
+                         int keep_first, const float* sinks, int page_size, int num_pages, void* stream);
 
 // The same attention on the matrix cores, bfloat16 only, head_dim and v_dim (the size of a value and of a
 // head's output: out [rows][nh * v_dim]) multiples of 16 up to 256.
@@ -153,7 +159,8 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,
                          int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
-                         int chunk, float softcap, int page_size, int num_pages, int heads_together, void* stream);
+                         int chunk, float softcap, int keep_first, const float* sinks, int page_size, int num_pages,
+                         int heads_together, void* stream);
 // Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
 // merged in order by the workgroup that finishes last. partial: float32 workspace
 // [rows][heads][max_splits][v_dim + 4]; max_context: an upper bound on position + 1 of every
@@ -164,8 +171,8 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
 int fw_attention_decode(const void* q, void* out, float* partial, int max_splits, int max_context,
                         const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                        int head_dim, int v_dim, float scale, int window, int chunk, float softcap, int page_size, int num_pages,
-                        void* stream);
+                        int head_dim, int v_dim, float scale, int window, int chunk, float softcap, int keep_first,
+                        const float* sinks, int page_size, int num_pages, void* stream);
 
 // The same with the work of fw_qk_norm_rope_kv_write in front of it, in one kernel: qkv float32
 // [rows][(heads + kv_heads) * head_dim + kv_heads * v_dim] are the step's raw projections; every workgroup norms and
@@ -177,8 +184,8 @@ int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, cons
                               int tickets_len, void* k_pages,
                               void* v_pages, const int32_t* block_table, int table_stride, const int32_t* row_seg,
                               const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim,
-                              float scale, int window, int chunk, float softcap, int interleaved, int page_size, int num_pages,
-                              void* stream);
+                              float scale, int window, int chunk, float softcap, int interleaved, int q_only, int keep_first,
+                              const float* sinks, int page_size, int num_pages, void* stream);
 
 // ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
 // advance[r] += 1 if that is not null; workspace: rows * 64 64-bit words
@@ -245,7 +252,7 @@ int fw_gated_delta_rule(const float* records, float* state, float* out, const in
                         int slots, void* stream);
 // out[r][h][j] = o[r][h][j] * rsqrt(mean_j o[r][h]^2 + eps) * weight[j] * act(gate[r][h vd + j]);
 // act is the sigmoid, or with gate_silu z * sigmoid(z)
-int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight,
+int fw_gated_head_norm(const float* o, const void* gate, int gate_dtype, int gate_stride, const float* weight, int weight_per_head,
                        void* out, int out_dtype, int rows, int heads, int vdim, float eps, int gate_silu, void* stream);
 
 // ---- sublayers whose output is normed ------------------------------------------------------------
@@ -280,6 +287,40 @@ int fw_latent_norm_write(const float* raw, int raw_stride, int col0, const float
 // out [rows][heads N].
 int fw_head_linear(const void* in, int in_dtype, int in_stride, const void* w, int w_dtype, const float* gate, int gate_stride,
                    void* out, int out_dtype, int rows, int heads, int N, int K, void* stream);
+
+// ---- a recurrence with a decay per key channel formed by the token ("wkv") --------------------------------
+// Token shift: h = rmsnorm(x) * (w or 1 + w) (norm_weight null: h = x); out[s][r] = h[r] + (h[r - 1] - h[r]) * mu[s],
+// s < mixes, out [mixes][rows][hidden] of out_dtype; the row before a segment's first is last[slot] (float32
+// [slots][hidden]), which is moved on to the h of the segment's last row.
+int fw_token_shift_mix(const float* x, const float* norm_weight, float eps, int one_centered, const float* mu, int mixes,
+                       float* last, int slots, const int32_t* row_seg, const int32_t* seg_row0, const int32_t* seg_slot,
+                       void* out, int out_dtype, int rows, int segments, int hidden, void* stream);
+// out = tanh(x): float32 in, out_dtype out
+int fw_tanh_rows(const float* x, void* out, int out_dtype, long long count, void* stream);
+// Per head: o_t = S^T r_t + (r_t . (u k_t)) v_t; S <- diag(exp(-exp(a_t + w0))) S + k_t v_t^T. r, k, v float32 rows of
+// rkv_stride floats (heads * dim used), a rows of a_stride; w0 [heads * dim], u [heads * dim]; state float32
+// [slots][heads][dim (key)][dim (value)]; out float32 [rows][heads * dim].
+int fw_wkv_recurrence(const float* r, const float* k, const float* v, int rkv_stride, const float* a, int a_stride,
+                      const float* w0, const float* u, float* state, int slots, float* out, const int32_t* seg_row0,
+                      const int32_t* seg_slot, int rows, int segments, int heads, int dim, void* stream);
+
+// ---- a mixture of feed-forward units chosen per token ------------------------------------------------------
+// chosen / weight [rows][top]: the `top` largest of logits[r] + bias (float32 [rows][experts]; ties: the lowest
+// id; bias may be null), largest first, and the softmax over those alone.
+int fw_moe_route(const float* logits, const float* bias, int32_t* chosen, float* weight, int rows, int experts, int top,
+                 void* stream);
+// The pairs (row, choice) sorted by expert, in the order of the pairs within an expert: expert_begin
+// [experts + 1], place_row [rows * top] (the row of each place), pair_place [rows * top] (the place of each pair).
+int fw_moe_arrange(const int32_t* chosen, int32_t* expert_begin, int32_t* place_row, int32_t* pair_place, int rows, int experts,
+                   int top, void* stream);
+// out[place] = a[place_row ? place_row[place] : place] . w[expert of place]^T; w [experts][N][K], or with
+// gated [experts][2 N][K] (gate rows, then up rows) and out = silu(gate) * up. out [places][N].
+int fw_grouped_gemm(const void* a, int a_dtype, const int32_t* place_row, const void* w, int w_dtype,
+                    const int32_t* expert_begin, void* out, int out_dtype, int gated, int places, int experts, int N, int K,
+                    void* stream);
+// x[r] += sum_j weight[r][j] * y[pair_place[r][j]], j in order; float32
+int fw_moe_combine(float* x, const float* y, const float* weight, const int32_t* pair_place, int rows, int top, int hidden,
+                   void* stream);
 
 #ifdef __cplusplus
 }

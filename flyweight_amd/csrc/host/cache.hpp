@@ -55,6 +55,7 @@ struct Group {
     // Which keys a sequence still needs: 0: every key; w > 0: the last w (a sliding window); -c < 0: those of
     // the chunk of c positions that the next token falls into (chunks counted from position 0).
     int window;
+    int keep_first = 0;     // beside a window: the first keys of a sequence stay needed, and so do their pages
     Pool pool;
     std::unordered_map<int64_t, std::vector<int>> tables;   // request -> page per block (NO_PAGE once given back)
     Group(int window_, int pages) : window(window_), pool(pages) {}
@@ -103,11 +104,21 @@ public:
     // Blocks before this one hold only keys the window has passed (or that lie before the chunk
     // of the next token) once the sequence is `length` tokens long (the next query sits at
     // position `length`).
+    // (A group that keeps first keys: the blocks that hold them are needed too, see still_needed.)
     int first_needed_block(const Group& group, int length) const {
         if (group.window == 0) return 0;
         if (group.window < 0) return (length - length % -group.window) / page_size_;
         const int first_key = length - group.window + 1 > 0 ? length - group.window + 1 : 0;
         return first_key / page_size_;
+    }
+
+    bool still_needed(const Group& group, int block, int length) const {
+        return block >= first_needed_block(group, length) || (group.window > 0 && block * page_size_ < group.keep_first);
+    }
+    void set_keep_first(int g, int keys) {
+        if (keys < 0) throw std::invalid_argument("the number of first keys to keep must not be negative");
+        if (!live_.empty()) throw AccountingError("what a group keeps is set before any request is live");
+        groups_.at(g).keep_first = keys;
     }
 
     bool is_live(int64_t request) const { return live_.count(request) != 0; }
@@ -188,7 +199,7 @@ public:
             std::vector<int>& table = group.tables[request];
             const int passed = first_needed_block(group, new_length);
             for (int block = 0; block < passed && block < (int)table.size(); ++block)
-                if (table[block] != NO_PAGE) {
+                if (table[block] != NO_PAGE && !still_needed(group, block, new_length)) {
                     group.pool.free(table[block]);
                     table[block] = NO_PAGE;
                 }
@@ -205,8 +216,8 @@ public:
         if (token_count < state.length)
             for (const Group& group : groups_) {
                 const std::vector<int>& table = group.tables.at(request);
-                for (int block = first_needed_block(group, token_count); block < keep && block < (int)table.size(); ++block)
-                    if (table[block] == NO_PAGE)
+                for (int block = 0; block < keep && block < (int)table.size(); ++block)
+                    if (table[block] == NO_PAGE && still_needed(group, block, token_count))
                         throw std::invalid_argument("request " + std::to_string(request) + " cannot be cut back to " +
                                                     std::to_string(token_count) + " tokens: its window has passed keys it would need");
             }

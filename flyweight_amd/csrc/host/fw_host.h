@@ -38,6 +38,8 @@ void* fwh_cache_create(int num_groups, const int* windows, int num_pages, int ma
 void* fwh_cache_create_sized(int num_groups, const int* windows, const int* pages, int max_requests, int page_size,
                              int max_pages_per_request);
 void fwh_cache_destroy(void* cache);
+// beside a window: the pages that hold a sequence's first `keys` keys are never given back while it lives
+int fwh_cache_set_keep_first(void* cache, int group, int keys);
 void* fwh_cache_group_pool(void* cache, int group);     // borrowed: lives as long as the cache
 void* fwh_cache_slot_pool(void* cache);
 int fwh_cache_admit(void* cache, int64_t request);      // the slot; FWH_OUT_OF_PAGES when no slot is free

@@ -38,7 +38,7 @@ int copy_ids(const std::vector<fwh::Request*>& from, int64_t* to) {
 extern "C" {
 
 const char* fwh_last_error(void) { return last_error.c_str(); }
-int fwh_abi_version(void) { return 5; }
+int fwh_abi_version(void) { return 6; }
 
 // ---- pools ---------------------------------------------------------------------------------
 void* fwh_pool_create(int size) {
@@ -75,6 +75,9 @@ void* fwh_cache_create_sized(int num_groups, const int* windows, const int* page
         return 0;
     });
     return made;
+}
+int fwh_cache_set_keep_first(void* cache, int group, int keys) {
+    return guarded([&] { cache_of(cache)->set_keep_first(group, keys); return 0; });
 }
 void fwh_cache_destroy(void* cache) { delete cache_of(cache); }
 void* fwh_cache_group_pool(void* cache, int group) {

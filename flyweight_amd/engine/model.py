@@ -49,6 +49,8 @@ class CausalLM:
     def tensors(self) -> Dict[str, TensorDecl]:
         spec = self.spec
         declared: Dict[str, TensorDecl] = {spec.embedding_name: TensorDecl((spec.vocab_size, spec.hidden_size))}
+        if spec.position_table_name is not None:        # a learned vector per position: as many as the model allows positions
+            declared[spec.position_table_name] = TensorDecl((spec.max_positions, spec.hidden_size))
         for block in self.layers:
             declared.update(block.tensors())
         declared.update(self.final_norm.tensors())
@@ -60,6 +62,8 @@ class CausalLM:
         self.dtype, self.device = dtype, device
         ops.prepare_device(device)
         self.embedding = tensors[self.spec.embedding_name]
+        name = self.spec.position_table_name
+        self.position_table = tensors[name] if name is not None else None
         head = self.embedding if self.spec.lm_head_name is None else tensors[self.spec.lm_head_name]
         self.head = Linear(head)
         for block in self.layers:
@@ -80,7 +84,14 @@ class CausalLM:
             if need is None:
                 continue
             if entry.cache in needs and needs[entry.cache] != need:
-                raise ConfigError(f"cache entry {entry.cache} is shared by layers with different needs")
+                # a layer that reads another's keys and values through a mask of its own: the entry keeps
+                # what either still sees
+                if not hasattr(need, "shared_with") or not hasattr(needs[entry.cache], "shared_with"):
+                    raise ConfigError(f"cache entry {entry.cache} is shared by layers with different needs")
+                try:
+                    need = needs[entry.cache].shared_with(need)
+                except ValueError as error:
+                    raise ConfigError(f"cache entry {entry.cache}: {error}") from None
             needs[entry.cache] = need
         return needs
 
@@ -105,7 +116,9 @@ class CausalLM:
     def forward(self, ctx, cache) -> Optional[torch.Tensor]:
         """Runs the rows of ``ctx`` through every scheduled layer; returns float32 logits
         [wanted, vocab] for ``ctx.want_rows`` (None when nothing is wanted)."""
-        x = ops.embed_rows(self.embedding, ctx.token_ids, scale=self.spec.embedding_scale)
+        # a learned vector per position joins the token's row in the same kernel, not scaled
+        x = ops.embed_rows(self.embedding, ctx.token_ids, scale=self.spec.embedding_scale, places_table=self.position_table,
+                           places=ctx.encoding_pos if self.position_table is not None else None)
         schedule = self.spec.schedule
         # A step of single tokens: the final norm reads every row as it is, like a layer's first norm, so
         # the last layer's last product may prepare it; rows that nobody wants cost the head nothing

@@ -20,7 +20,7 @@ F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256          # of the matrix-core attention kernels
 MAX_PLAIN_HEAD_DIM = 512    # of the plain attention kernels, which serve what the others do not take
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _lib = None
 
@@ -174,10 +174,19 @@ def _want(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
 
 
 # ---------------------------------------------------------------------------------------
-def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0) -> torch.Tensor:
-    _dev(table, ids, out)
+def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None, scale: float = 1.0,
+               places_table: Optional[torch.Tensor] = None, places: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """table[ids] * scale as float32 rows; with ``places_table`` and ``places`` (int32, one per row, checked against
+    the table by the caller) plus places_table[places], not scaled."""
+    _dev(table, ids, out, places_table, places)
     _want(ids, torch.int32, "ids")
     vocab, hidden = table.shape
+    if (places_table is None) != (places is None):
+        raise KernelError("embed_rows: a table of places and the rows' places come together")
+    if places is not None:
+        _want(places, torch.int32, "places")
+        if places_table.dim() != 2 or places_table.shape[1] != hidden or places.numel() < ids.numel():
+            raise KernelError(f"embed_rows: the table of places is {tuple(places_table.shape)} beside rows of {hidden}, {places.numel()} places for {ids.numel()} rows")
     rows = ids.numel()
     if out is None:
         out = torch.empty((rows, hidden), dtype=torch.float32, device=table.device)
@@ -185,7 +194,8 @@ def embed_rows(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tenso
     if out.shape != (rows, hidden):
         raise KernelError(f"embed_rows: out is {tuple(out.shape)}, expected {(rows, hidden)}")
     _check(library().fw_embed_rows(_p(table), _code(table.dtype), _p(ids), _p(out), rows, hidden, vocab,
-                                   ctypes.c_float(scale), _stream()))
+                                   ctypes.c_float(scale), _p(places_table), _code(places_table.dtype) if places_table is not None else F32,
+                                   _p(places), places_table.shape[0] if places_table is not None else 0, _stream()))
     return out
 
 
@@ -330,15 +340,16 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int,
                           k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                           row_seg: torch.Tensor, row_pos: torch.Tensor, write_kv: bool = True,
-                          v_dim: Optional[int] = None, interleaved: bool = False) -> torch.Tensor:
+                          v_dim: Optional[int] = None, interleaved: bool = False, q_only: bool = False) -> torch.Tensor:
     """The output and the cache take the pages' dtype; ``qkv`` may be float32 beside bfloat16 pages.
     ``v_dim``: the size of a value head where it is not ``head_dim``. ``interleaved``: channel 2i turns
     with channel 2i + 1 instead of channel i with channel i + rotary_dim / 2."""
     _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
     rows, width = qkv.shape
     v_dim = head_dim if v_dim is None else int(v_dim)
-    if width != (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim:
-        raise KernelError(f"qk_norm_rope: qkv width {width} != ({num_heads} + {num_kv_heads}) x {head_dim} + {num_kv_heads} x {v_dim}")
+    expected = num_heads * head_dim if q_only else (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim
+    if width != expected or (q_only and write_kv):
+        raise KernelError(f"qk_norm_rope: qkv width {width} != {expected} (queries alone: {q_only}; they bring nothing to store)")
     pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, k_pages.dtype, v_dim)
     for w in (q_norm_weight, k_norm_weight):
         if w is not None:
@@ -359,14 +370,27 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
     _check(library().fw_qk_norm_rope_kv_write(
         _p(qkv), _code(qkv.dtype), _p(q_out), _code(k_pages.dtype), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin),
         rotary_dim, _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg), _p(row_pos), rows,
-        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), int(interleaved), _stream()))
+        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), int(interleaved), int(q_only), _stream()))
     return q_out
+
+
+def _sinks(sinks: Optional[torch.Tensor], num_heads: int, keep_first: int, window: int, chunk: int):
+    """Checks what the mask and the softmax take beyond a window: ``keep_first`` first keys that stay seen
+    (beside a window only) and one more term exp(sinks[head]) in the denominator (float32 [heads])."""
+    if keep_first < 0 or (keep_first and chunk):
+        raise KernelError(f"attention: {keep_first} first keys are kept beside a window, not beside chunks")
+    if sinks is not None:
+        _dev(sinks)
+        _want(sinks, torch.float32, "sinks")
+        if sinks.shape != (num_heads,):
+            raise KernelError(f"attention: sinks are {tuple(sinks.shape)}, expected one per head ({num_heads})")
+    return int(keep_first) if window else 0, _p(sinks)
 
 
 def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                       scale: float, window: int = 0, v_dim: Optional[int] = None, chunk: int = 0,
-                      softcap: float = 0.0) -> torch.Tensor:
+                      softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``v_dim``: the size of a value head (and of a head's output) where it is not ``head_dim``.
     ``chunk`` > 0: a row sees only the keys of its own chunk of that many positions; ``softcap`` c > 0:
     score <- c tanh(score / c)."""
@@ -385,7 +409,7 @@ def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(library().fw_attention_generic(
         _p(q), _p(out), _code(q.dtype), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg),
         _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window), int(chunk),
-        ctypes.c_float(softcap), PAGE_SIZE, pages, _stream()))
+        ctypes.c_float(softcap), *_sinks(sinks, num_heads, keep_first, window, chunk), PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -879,12 +903,12 @@ def query_tiles(seg_row0):
     return tile_seg, tile_row0
 
 
-def decode_splits(max_context: int, window: int = 0, chunk: int = 0) -> int:
+def decode_splits(max_context: int, window: int = 0, chunk: int = 0, keep_first: int = 0) -> int:
     """Into how many workgroups at most the keys that a row sees are cut: runs of 4 pages."""
     blocks = (max_context + PAGE_SIZE - 1) // PAGE_SIZE
     span = min((n for n in (window, chunk) if n > 0), default=0)     # the most keys a row sees, where bounded
     if span > 0:
-        blocks = min(blocks, (span + PAGE_SIZE - 2) // PAGE_SIZE + 1)
+        blocks = min(blocks, (span + PAGE_SIZE - 2) // PAGE_SIZE + 1 + (keep_first + PAGE_SIZE - 1) // PAGE_SIZE)
     return max(1, (blocks + DECODE_SPLIT_PAGES - 1) // DECODE_SPLIT_PAGES)
 
 
@@ -892,7 +916,7 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                       v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
                       seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0,
                       heads_together: int = 0, out: Optional[torch.Tensor] = None, v_dim: Optional[int] = None,
-                      chunk: int = 0, softcap: float = 0.0) -> torch.Tensor:
+                      chunk: int = 0, softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the
     kernel's choice. Only the rows of the given tiles are written (into ``out`` if given)."""
     _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
@@ -914,7 +938,8 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(library().fw_attention_prefill(
         _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
         tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
-        int(window), int(chunk), ctypes.c_float(softcap), PAGE_SIZE, pages, int(heads_together), _stream()))
+        int(window), int(chunk), ctypes.c_float(softcap), *_sinks(sinks, num_heads, keep_first, window, chunk), PAGE_SIZE, pages,
+        int(heads_together), _stream()))
     return out
 
 
@@ -931,7 +956,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                      v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                      scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None,
                      decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
-                     softcap: float = 0.0) -> torch.Tensor:
+                     softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it).
     ``decode_work``: one int32 on the device, the runs of 4 pages that the rows see together (the
     sum of ceil((position + 1) / 256)): the kernel shares the work out by it (fewer, longer
@@ -947,7 +972,8 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    splits = decode_splits(max_context, window, chunk)
+    keep_first, sinks_at = _sinks(sinks, num_heads, keep_first, window, chunk)
+    splits = decode_splits(max_context, window, chunk, keep_first)
     partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty((rows, num_heads * v_dim), dtype=q.dtype, device=q.device)
@@ -959,7 +985,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _p(q), _p(out), _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
         _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
-        int(window), int(chunk), ctypes.c_float(softcap), PAGE_SIZE, pages, _stream()))
+        int(window), int(chunk), ctypes.c_float(softcap), keep_first, sinks_at, PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -969,7 +995,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
                            v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                            scale: float, max_context: int, window: int = 0, write_kv: bool = True,
                            decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
-                           softcap: float = 0.0, interleaved: bool = False) -> torch.Tensor:
+                           softcap: float = 0.0, interleaved: bool = False, q_only: bool = False, keep_first: int = 0,
+                           sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One row per request, from the step's raw projections ``qkv`` (float32 [rows, (heads + 2 kv
     heads) * head_dim]): per-head norm and rotation of queries and keys, the new keys and values
     into their pages, and the split-key attention, in one kernel. Returns bfloat16 [rows, heads *
@@ -978,8 +1005,9 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
     _want(qkv, torch.float32, "qkv")
     rows, width = qkv.shape
     v_dim = head_dim if v_dim is None else int(v_dim)
-    if width != (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim:
-        raise KernelError(f"attention_decode_fused: qkv width {width} != ({num_heads} + {num_kv_heads}) x {head_dim} + {num_kv_heads} x {v_dim}")
+    expected = num_heads * head_dim if q_only else (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim
+    if width != expected or (q_only and write_kv):
+        raise KernelError(f"attention_decode_fused: qkv width {width} != {expected} (queries alone: {q_only}; they bring nothing to store)")
     pages = _check_pages(k_pages, v_pages, num_kv_heads, head_dim, torch.bfloat16, v_dim)
     for w in (q_norm_weight, k_norm_weight):
         if w is not None:
@@ -995,7 +1023,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    splits = decode_splits(max_context, window, chunk)
+    keep_first, sinks_at = _sinks(sinks, num_heads, keep_first, window, chunk)
+    splits = decode_splits(max_context, window, chunk, keep_first)
     partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=qkv.device)
     out = torch.empty((rows, num_heads * v_dim), dtype=torch.bfloat16, device=qkv.device)
     group = num_heads // num_kv_heads
@@ -1004,7 +1033,7 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
         _p(qkv), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim), int(write_kv), _p(out),
         _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window),
-        int(chunk), ctypes.c_float(softcap), int(interleaved), PAGE_SIZE, pages, _stream()))
+        int(chunk), ctypes.c_float(softcap), int(interleaved), int(q_only), keep_first, sinks_at, PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -1018,7 +1047,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0,
               tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None,
               decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
-              softcap: float = 0.0) -> torch.Tensor:
+              softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
     kernel for segments of one row (all of them, or those a mixed step begins with: a single row
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
@@ -1031,7 +1060,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                                 ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work, v_dim=v_dim,
-                                chunk=chunk, softcap=softcap)
+                                chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
     if fast:
         if tile_seg is None or tile_row0 is None:
             raise KernelError("attention: the tiled kernel needs the step's query tiles")
@@ -1045,16 +1074,17 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
         if single == 0:
             return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, tile_seg,
                                      tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together, v_dim=v_dim,
-                                     chunk=chunk, softcap=softcap)
+                                     chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
         out = torch.empty((q.shape[0], num_heads * v_dim), dtype=q.dtype, device=q.device)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                          ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work, v_dim=v_dim,
-                         chunk=chunk, softcap=softcap)
+                         chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
-                                 heads_together=together, out=out, v_dim=v_dim, chunk=chunk, softcap=softcap)
+                                 heads_together=together, out=out, v_dim=v_dim, chunk=chunk, softcap=softcap,
+                                 keep_first=keep_first, sinks=sinks)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                             ctx.row_pos, scale, window, v_dim=v_dim, chunk=chunk, softcap=softcap)
+                             ctx.row_pos, scale, window, v_dim=v_dim, chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
 
 
 # ---- the gated delta rule -----------------------------------------------------------------------------
@@ -1129,6 +1159,7 @@ def gated_delta_rule(records: torch.Tensor, state: torch.Tensor, seg_row0: torch
 
 def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, heads: int, vdim: int, eps: float,
                     out_dtype: torch.dtype, gate_silu: bool = False) -> torch.Tensor:
+    # ``weight`` [vdim] serves every head; [heads * vdim] gives each head its own
     """Per head: o / rms(o) * weight * sigmoid(gate) (``gate_silu``: times gate * sigmoid(gate)); ``o`` float32 [rows, heads vdim], ``gate``
     [rows, heads vdim] (float32, or bfloat16 beside a bfloat16 output; a view of wider rows will do)."""
     _dev(o, weight)
@@ -1136,10 +1167,11 @@ def gated_head_norm(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, h
     _want(o, torch.float32, "o")
     _want(weight, torch.float32, "weight")
     rows = o.shape[0]
-    if o.shape != (rows, heads * vdim) or gate.shape != o.shape or weight.shape != (vdim,) or not o.is_contiguous() or gate.stride(1) != 1:
+    per_head = weight.shape == (heads * vdim,) and heads > 1
+    if o.shape != (rows, heads * vdim) or gate.shape != o.shape or (weight.shape != (vdim,) and not per_head) or not o.is_contiguous() or gate.stride(1) != 1:
         raise KernelError(f"gated_head_norm: o {tuple(o.shape)}, gate {tuple(gate.shape)}, weight {tuple(weight.shape)} do not fit {heads} x {vdim}")
     out = torch.empty((rows, heads * vdim), dtype=out_dtype, device=o.device)
-    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), gate.stride(0) if rows > 1 else max(heads * vdim, gate.stride(0)), _p(weight), _p(out), _code(out_dtype), rows,
+    _check(library().fw_gated_head_norm(_p(o), _p(gate), _code(gate.dtype), gate.stride(0) if rows > 1 else max(heads * vdim, gate.stride(0)), _p(weight), int(per_head), _p(out), _code(out_dtype), rows,
                                         heads, vdim, ctypes.c_float(eps), int(gate_silu), _stream()))
     return out
 
@@ -1303,3 +1335,138 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: 
                                     stride(gate, heads * N) if gate is not None else 0, _p(out), _code(out_dtype), rows, heads, N, K,
                                     _stream()))
     return out
+
+
+# ---- a recurrence with a decay per key channel formed by the token ("wkv") --------------------------------------
+def token_shift_mix(x: torch.Tensor, norm_weight: Optional[torch.Tensor], eps: float, one_centered: bool, mu: torch.Tensor,
+                    last: torch.Tensor, row_seg: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """h = rmsnorm(x) * weight (``norm_weight`` None: h = x); returns [mixes, rows, hidden] = h + (h of the row before - h)
+    * mu[s]. ``last`` float32 [slots, hidden]: the h of each request's last row so far, read for a segment's first
+    row and moved on."""
+    _dev(x, norm_weight, mu, last, row_seg, seg_row0, seg_slot)
+    _want(x, torch.float32, "x")
+    _want(mu, torch.float32, "mu")
+    _want(last, torch.float32, "last")
+    rows, hidden = x.shape
+    if mu.dim() != 2 or mu.shape[1] != hidden or last.dim() != 2 or last.shape[1] != hidden:
+        raise KernelError(f"token_shift_mix: mu {tuple(mu.shape)} / last {tuple(last.shape)} beside rows of {hidden}")
+    if norm_weight is not None and (norm_weight.dtype != torch.float32 or norm_weight.shape != (hidden,)):
+        raise KernelError("token_shift_mix: the norm's weight is float32 [hidden]")
+    for name, t, n in (("row_seg", row_seg, rows), ("seg_row0", seg_row0, segments + 1), ("seg_slot", seg_slot, segments)):
+        _want(t, torch.int32, name)
+        if t.numel() < n:
+            raise KernelError(f"token_shift_mix: {name} holds {t.numel()} entries, needs {n}")
+    out = torch.empty((mu.shape[0], rows, hidden), dtype=out_dtype, device=x.device)
+    _check(library().fw_token_shift_mix(_p(x), _p(norm_weight), ctypes.c_float(eps), int(one_centered), _p(mu), mu.shape[0], _p(last),
+                                        last.shape[0], _p(row_seg), _p(seg_row0), _p(seg_slot), _p(out), _code(out_dtype), rows,
+                                        int(segments), hidden, _stream()))
+    return out
+
+
+def tanh_rows(x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    _dev(x)
+    _want(x, torch.float32, "x")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _check(library().fw_tanh_rows(_p(x), _p(out), _code(out_dtype), ctypes.c_longlong(x.numel()), _stream()))
+    return out
+
+
+def wkv_recurrence(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.Tensor, w0: torch.Tensor, u: torch.Tensor,
+                   state: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int, heads: int, dim: int) -> torch.Tensor:
+    """Per head o_t = S^T r_t + (r_t . (u k_t)) v_t, then S <- diag(exp(-exp(a_t + w0))) S + k_t v_t^T, over each segment's rows
+    in order. ``r``, ``k``, ``v`` float32 [rows, heads dim] with one row stride (views of wider rows will do), ``a``
+    likewise; ``state`` float32 [slots, heads, dim, dim] is read and moved on. Returns float32 [rows, heads dim]."""
+    _dev(w0, u, state, seg_row0, seg_slot)
+    rows = r.shape[0]
+    width = heads * dim
+    for name, t in (("r", r), ("k", k), ("v", v), ("a", a)):
+        _dev_rows(t, name)
+        _want(t, torch.float32, name)
+        if t.shape != (rows, width):
+            raise KernelError(f"wkv_recurrence: {name} is {tuple(t.shape)}, expected {(rows, width)}")
+
+    def stride(t):
+        return t.stride(0) if rows > 1 else max(width, t.stride(0))
+
+    if not (stride(r) == stride(k) == stride(v)):
+        raise KernelError("wkv_recurrence: r, k and v have one row stride")
+    for name, t in (("w0", w0), ("u", u)):
+        _want(t, torch.float32, name)
+        if t.numel() != width:
+            raise KernelError(f"wkv_recurrence: {name} holds {t.numel()} values, expected {width}")
+    _want(state, torch.float32, "state")
+    if state.dim() != 4 or state.shape[1:] != (heads, dim, dim):
+        raise KernelError(f"wkv_recurrence: the state is {tuple(state.shape)}, expected [slots, {heads}, {dim}, {dim}]")
+    for name, t, n in (("seg_row0", seg_row0, segments + 1), ("seg_slot", seg_slot, segments)):
+        _want(t, torch.int32, name)
+        if t.numel() < n:
+            raise KernelError(f"wkv_recurrence: {name} holds {t.numel()} entries, needs {n}")
+    out = torch.empty((rows, width), dtype=torch.float32, device=r.device)
+    _check(library().fw_wkv_recurrence(_p(r), _p(k), _p(v), stride(r), _p(a), stride(a), _p(w0), _p(u), _p(state), state.shape[0], _p(out),
+                                       _p(seg_row0), _p(seg_slot), rows, int(segments), heads, dim, _stream()))
+    return out
+
+
+# ---- a mixture of feed-forward units chosen per token ------------------------------------------------------------
+def moe_route(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+    """(chosen int32 [rows, top], weight float32 [rows, top]): the ``top`` largest of logits + bias per row, largest
+    first (ties: the lowest id), and the softmax over those alone."""
+    _dev(logits, bias)
+    _want(logits, torch.float32, "logits")
+    rows, experts = logits.shape
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (experts,)):
+        raise KernelError("moe_route: the bias is float32 [experts]")
+    chosen = torch.empty((rows, top), dtype=torch.int32, device=logits.device)
+    weight = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
+    _check(library().fw_moe_route(_p(logits), _p(bias), _p(chosen), _p(weight), rows, experts, int(top), _stream()))
+    return chosen, weight
+
+
+def moe_arrange(chosen: torch.Tensor, experts: int):
+    """The pairs (row, choice) sorted by expert, an expert's pairs in their order: (expert_begin int32 [experts + 1],
+    place_row int32 [pairs], pair_place int32 [rows, top])."""
+    _dev(chosen)
+    _want(chosen, torch.int32, "chosen")
+    rows, top = chosen.shape
+    expert_begin = torch.empty((experts + 1,), dtype=torch.int32, device=chosen.device)
+    place_row = torch.empty((rows * top,), dtype=torch.int32, device=chosen.device)
+    pair_place = torch.empty((rows, top), dtype=torch.int32, device=chosen.device)
+    _check(library().fw_moe_arrange(_p(chosen), _p(expert_begin), _p(place_row), _p(pair_place), rows, int(experts), top, _stream()))
+    return expert_begin, place_row, pair_place
+
+
+def grouped_gemm(a: torch.Tensor, place_row: Optional[torch.Tensor], w: torch.Tensor, expert_begin: torch.Tensor, places: int,
+                 gated: bool, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[place] = a[place_row[place]] . w[expert of place]^T (``place_row`` None: a[place]); ``w`` [experts, N, K], or
+    with ``gated`` [experts, 2 N, K] (gate rows, then up rows) and out = silu(gate) * up. Returns [places, N]."""
+    _dev(a, place_row, w, expert_begin)
+    experts, n_rows, K = w.shape
+    N = n_rows // 2 if gated else n_rows
+    if a.dim() != 2 or a.shape[1] != K or (gated and n_rows % 2) or expert_begin.numel() != experts + 1:
+        raise KernelError(f"grouped_gemm: a is {tuple(a.shape)}, w {tuple(w.shape)}, {expert_begin.numel()} expert bounds")
+    _want(expert_begin, torch.int32, "expert_begin")
+    if place_row is not None:
+        _want(place_row, torch.int32, "place_row")
+        if place_row.numel() < places:
+            raise KernelError("grouped_gemm: fewer rows named than places")
+    elif a.shape[0] < places:
+        raise KernelError("grouped_gemm: fewer rows than places")
+    out = torch.empty((places, N), dtype=out_dtype, device=a.device)
+    _check(library().fw_grouped_gemm(_p(a), _code(a.dtype), _p(place_row), _p(w), _code(w.dtype), _p(expert_begin), _p(out),
+                                     _code(out_dtype), int(gated), int(places), experts, N, K, _stream()))
+    return out
+
+
+def moe_combine_(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, pair_place: torch.Tensor) -> torch.Tensor:
+    """x[row] += sum over the row's choices, in their order, of weight[row, j] * y[pair_place[row, j]]; float32."""
+    _dev(x, y, weight, pair_place)
+    for name, t in (("x", x), ("y", y), ("weight", weight)):
+        _want(t, torch.float32, name)
+    _want(pair_place, torch.int32, "pair_place")
+    rows, hidden = x.shape
+    top = weight.shape[1]
+    if weight.shape != (rows, top) or pair_place.shape != (rows, top) or y.shape != (rows * top, hidden):
+        raise KernelError(f"moe_combine: x {tuple(x.shape)}, y {tuple(y.shape)}, weight {tuple(weight.shape)}, places {tuple(pair_place.shape)}")
+    _check(library().fw_moe_combine(_p(x), _p(y), _p(weight), _p(pair_place), rows, top, hidden, _stream()))
+    return x

@@ -5,7 +5,12 @@ head_dim shared by all heads); position encoding on q and k; k and v appended to
 cache; scores q.k * softmax_scale (1 / sqrt(head_dim) unless given) over the cached keys the row
 may see (causal, optionally only the last ``window``: itself and the window - 1 before it; with
 ``chunk`` only those of the row's own chunk of that many positions, chunks counted from position 0 of
-the sequence), optionally capped softly (``score_softcap`` c: c tanh(score / c)), softmax in float32, weighted sum of values; out = W_o o. Values may have a size of their own
+the sequence), optionally capped softly (``score_softcap`` c: c tanh(score / c)), softmax in float32, weighted sum of values; out = W_o o.
+Beside a window ``keep_first`` n keeps the first n keys of the sequence seen wherever the window stands
+(row i sees key j <= i if i - j < window or j < n). ``sink`` gives every head a learned number s (tensor
+``names["sink"]``, [heads]) whose exp(s) joins the softmax's denominator: a term with no key and no value, not
+scaled. ``shared_kv``: the layer has no key and value projections; it reads the cache entry of another layer
+(the schedule names it and says that this layer does not write it), with its own queries and mask. Values may have a size of their own
 (``v_head_dim``); the output of a head has that size.
 Query head i reads kv head i // (num_heads / num_kv_heads). Formulas as the reference's
 LFM2 attention branch computes them (native/src/v2_runtime.cpp:28429-28478).
@@ -25,7 +30,7 @@ from ..weights.loader import TensorDecl
 from .base import Mixer, build_part, register_mixer
 from .linear import Linear
 
-_DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "q_norm": "q_norm", "k_norm": "k_norm"}
+_DEFAULT_NAMES = {"q": "q_proj", "k": "k_proj", "v": "v_proj", "o": "o_proj", "q_norm": "q_norm", "k_norm": "k_norm", "sink": "sink"}
 
 
 class QueryTileArrays:
@@ -90,6 +95,9 @@ class GQAttention(QueryTileArrays, Mixer):
         self.window = spec.get("window")
         self.chunk = int(spec.get("chunk") or 0)
         self.softcap = float(spec.get("score_softcap") or 0.0)
+        self.keep_first = int(spec.get("keep_first") or 0)
+        self.has_sink = bool(spec.get("sink", False))
+        self.shared_kv = bool(spec.get("shared_kv", False))
         self.scale = float(spec.get("softmax_scale", self.head_dim ** -0.5))
         self.bias = bool(spec.get("bias", False))
         self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
@@ -106,10 +114,15 @@ class GQAttention(QueryTileArrays, Mixer):
             raise ConfigError("an attention window must be positive (or None for all keys)")
         if self.chunk < 0 or self.softcap < 0:
             raise ConfigError("an attention chunk and a soft cap on the scores must be positive (or 0 / None for none)")
+        if self.keep_first < 0 or (self.keep_first and self.chunk):
+            raise ConfigError("first keys are kept beside a window (a non-negative number of them), not beside chunks")
+        if self.shared_kv and (self.bias or self.qk_norm):
+            raise ConfigError("a layer that reads another layer's keys and values has no biases and no per-head norms here")
 
     def cache_need(self):
         return PagedKV(self.num_kv_heads, self.head_dim, None if self.window is None else int(self.window),
-                       None if self.v_head_dim == self.head_dim else self.v_head_dim, self.chunk or None)
+                       None if self.v_head_dim == self.head_dim else self.v_head_dim, self.chunk or None,
+                       self.keep_first if self.window is not None else 0)
 
     def _name(self, which: str, leaf: str = "weight") -> str:
         if leaf == "weight":
@@ -124,6 +137,10 @@ class GQAttention(QueryTileArrays, Mixer):
             self._name("v"): TensorDecl((self.num_kv_heads * self.v_head_dim, self.hidden)),
             self._name("o"): TensorDecl((self.hidden, self.num_heads * self.v_head_dim)),
         }
+        if self.shared_kv:
+            del declared[self._name("k")], declared[self._name("v")]
+        if self.has_sink:
+            declared[self._name("sink")] = TensorDecl((self.num_heads,), "vector", "bias")
         if self.bias:
             declared[self._name("q", "bias")] = TensorDecl((q_width,), "vector", "bias")
             declared[self._name("k", "bias")] = TensorDecl((kv_width,), "vector", "bias")
@@ -137,12 +154,16 @@ class GQAttention(QueryTileArrays, Mixer):
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
         self.position.bind(tensors, dtype, device)
-        q, k, v = (tensors[self._name(n)] for n in ("q", "k", "v"))
-        if not (q.dtype == k.dtype == v.dtype):
-            raise ConfigError(f"{self.prefix}: q, k and v projections are stored in different precisions")
-        # one operand for the three projections: rows are q heads, then k heads, then v heads
-        bias = torch.cat([tensors[self._name(n, "bias")] for n in ("q", "k", "v")]) if self.bias else None
-        self.qkv = Linear(torch.cat([q, k, v], dim=0), bias)
+        self.sinks = tensors[self._name("sink")] if self.has_sink else None
+        if self.shared_kv:
+            self.qkv = Linear(tensors[self._name("q")])        # the queries alone
+        else:
+            q, k, v = (tensors[self._name(n)] for n in ("q", "k", "v"))
+            if not (q.dtype == k.dtype == v.dtype):
+                raise ConfigError(f"{self.prefix}: q, k and v projections are stored in different precisions")
+            # one operand for the three projections: rows are q heads, then k heads, then v heads
+            bias = torch.cat([tensors[self._name(n, "bias")] for n in ("q", "k", "v")]) if self.bias else None
+            self.qkv = Linear(torch.cat([q, k, v], dim=0), bias)
         self.out = Linear(tensors[self._name("o")], tensors[self._name("o", "bias")] if self.bias else None)
         self.q_norm_weight = tensors[self._name("q_norm")] if self.qk_norm else None
         self.k_norm_weight = tensors[self._name("k_norm")] if self.qk_norm else None
@@ -158,6 +179,9 @@ class GQAttention(QueryTileArrays, Mixer):
         cos, sin = ctx.position_tables(self.position)
         interleaved = bool(getattr(self.position, "interleaved", False))
         own = ctx.step_arrays(self) if self.step_arrays_key() is not None else {}
+        if self.shared_kv and cache.writes:
+            raise ConfigError(f"{self.prefix}: the layer has no keys and values of its own; its schedule entry must read another's cache entry")
+        mask = {"keep_first": self.keep_first if self.window else 0, "sinks": self.sinks}
         if ctx.all_decode and ctx.num_rows <= self.FUSED_DECODE_ROWS and qkv.dtype == torch.float32 and self.step_arrays_key() is not None:
             # a few single-token segments on the matrix cores: norm, rotation, cache write and attention in one kernel
             return ops.attention_decode_fused(
@@ -165,15 +189,15 @@ class GQAttention(QueryTileArrays, Mixer):
                 cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table, ctx.row_seg, ctx.row_pos,
                 self.scale, ctx.max_context, int(self.window or 0), write_kv=cache.writes,
                 decode_work=own.get("decode_work"), v_dim=self.v_head_dim, chunk=self.chunk, softcap=self.softcap,
-                interleaved=interleaved)
+                interleaved=interleaved, q_only=self.shared_kv, **mask)
         q = ops.qk_norm_rope_kv_write(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.q_norm_weight, self.k_norm_weight,
             self.qk_norm_eps, cos, sin, self.position.rotary_dim, cache.k_pages, cache.v_pages, cache.block_table,
-            ctx.row_seg, ctx.row_pos, write_kv=cache.writes, v_dim=self.v_head_dim, interleaved=interleaved)
+            ctx.row_seg, ctx.row_pos, write_kv=cache.writes, v_dim=self.v_head_dim, interleaved=interleaved, q_only=self.shared_kv)
         return ops.attention(q, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
                              cache.block_table, ctx, self.scale, int(self.window or 0),
                              tile_seg=own.get("tile_seg"), tile_row0=own.get("tile_row0"), decode_work=own.get("decode_work"),
-                             v_dim=self.v_head_dim, chunk=self.chunk, softcap=self.softcap)
+                             v_dim=self.v_head_dim, chunk=self.chunk, softcap=self.softcap, **mask)
 
     def forward(self, h, residual, ctx, cache):
         return self.out.accumulate(self.attend(h, ctx, cache), residual, then=getattr(ctx, "upcoming_norm", None))

@@ -12,6 +12,10 @@ sublayer's OUTPUT, and m is a fixed factor. The feed-forward may be absent.
 and a norm behind every sublayer; then, where the layer has one, the tokens' own input
 (``parts/token_input.py``): x <- x + rms(y(x, token)) * w. The feed-forward may be absent. Every sum into
 x also forms what reads x next (the next norm's output, or x rounded) in the same kernel.
+
+
+``parallel_residual``: with h = norm1(x), x <- x + (mixer(h) + ffn(h)): one norm, and both sublayers read its
+output. The feed-forward may be absent.
 """
 
 from __future__ import annotations
@@ -199,3 +203,48 @@ class SandwichNormResidualBlock(Block):
         if self.token_input is not None:
             h = self._join(x, self.token_input.output(h, ctx), self.token_input, after, dtype)
         return NormedRows(after, h) if after is not None and h is not None else None
+
+
+@register_block("parallel_residual")
+class ParallelResidualBlock(Block):
+    """One norm whose output both sublayers read; their outputs join the residual stream together. Both
+    sublayers add into the float32 stream in their last product's epilogue, the mixer first."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.norm = build_part("norm", spec.mixer_norm)
+        self.mixer = build_part("mixer", spec.mixer)
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+        if spec.ffn_norm is not None:
+            raise ConfigError("the parallel arrangement has one norm; its feed-forward reads the mixer's")
+
+    def parts(self):
+        return tuple(part for part in (self.norm, self.mixer, self.ffn) if part is not None)
+
+    def first_norm(self):
+        return self.norm
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def graph_safe(self) -> bool:
+        position = getattr(self.mixer, "position", None)
+        return all(part.graph_safe for part in self.parts()) and (position is None or position.graph_safe)
+
+    def forward(self, x, ctx, cache, prepared=None, norm_after=None):
+        """``x`` [rows, hidden] float32 is updated in place."""
+        # Both sublayers must see the norm of x as it was: the feed-forward may not take the norm into a
+        # kernel of its own once the mixer has added to x, so it gets the rows normed beforehand unless the
+        # mixer needs none of them (a mixer that takes the norm into its own first kernel reads x before it
+        # writes it, and so does the feed-forward's product only if it runs first: it does not).
+        h = LazyNorm(self.norm, x, ctx, prepared=prepared if isinstance(prepared, NormedRows) else None)
+        normed = h.tensor() if self.ffn is not None or not getattr(self.mixer, "accepts_lazy_norm", False) else None
+        ctx.upcoming_norm = None
+        if normed is None or getattr(self.mixer, "wants_unnormed_rows", False):
+            self.mixer.forward(h, x, ctx, cache)
+        else:
+            self.mixer.forward(normed, x, ctx, cache)
+        if self.ffn is not None:
+            self.ffn.forward(normed, x, ctx)
+        return None

@@ -1,0 +1,101 @@
+"""A mixture of gated feed-forward units chosen per token.
+
+Router logits z = W_router h + b in float32 (h as the products read it); the ``top`` experts with the largest
+logits are chosen (ties: the lowest id) and weighted by the softmax over the chosen logits alone. An expert is
+W_down (silu(W_gate h) * (W_up h)) without biases; the output is the weighted sum of the chosen experts'
+outputs, summed in the order of the choices. ``shared_intermediate_size``: one more unit of that width runs for
+every token and is added. The experts' weights lie stacked ([experts, 2 ff, hidden] gate rows then up rows,
+[experts, hidden, ff]); a step sorts its (token, choice) pairs by expert on the device and runs each expert's
+pairs as tiles of one grouped product, so nothing crosses to the host and a decode step can be recorded.
+"""
+
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..config.spec import ConfigError, PartSpec
+from ..kernels import ops
+from ..weights.loader import TensorDecl
+from .base import FeedForward, build_part, register_feed_forward
+from .norm import LazyNorm
+
+_DEFAULT_NAMES = {"router": "router", "router_bias": "router.b", "expert": "e{index}.", "gate": "gate", "up": "up", "down": "down",
+                  "shared": "shared."}
+
+
+@register_feed_forward("moe_swiglu")
+class MoeSwiGLU(FeedForward):
+    graph_safe = True
+    accepts_lazy_norm = True        # handed on to the shared unit, whose first product can take the norm
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.hidden = int(spec["hidden_size"])
+        self.experts = int(spec["num_experts"])
+        self.top = int(spec["top"])
+        self.intermediate = int(spec["intermediate_size"])
+        self.shared_intermediate = int(spec.get("shared_intermediate_size") or 0)
+        self.router_bias = bool(spec.get("router_bias", True))
+        self.names = {**_DEFAULT_NAMES, **dict(spec.get("names", {}))}
+        if not 1 <= self.top <= self.experts or self.experts > 1024 or self.top > 64:
+            raise ConfigError(f"a mixture of {self.experts} experts (at most 1,024) with {self.top} a token (at most 64)")
+        self.shared = None
+        if self.shared_intermediate:
+            self.shared = build_part("ffn", PartSpec("swiglu", {
+                "hidden_size": self.hidden, "intermediate_size": self.shared_intermediate,
+                "names": {which: self.names[which] for which in ("gate", "up", "down")}, "weight_suffix": ""},
+                prefix=self.prefix + self.names["shared"]))
+
+    def sub_parts(self):
+        return (self.shared,) if self.shared is not None else ()
+
+    def _expert(self, index: int, which: str) -> str:
+        return self.prefix + self.names["expert"].format(index=index) + self.names[which]
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        D, F = self.hidden, self.intermediate
+        # the router decides in float32: its weights are widened once, when they are loaded
+        declared = {self.prefix + self.names["router"]: TensorDecl((self.experts, D), "vector", "matrix")}
+        if self.router_bias:
+            declared[self.prefix + self.names["router_bias"]] = TensorDecl((self.experts,), "vector", "bias")
+        for index in range(self.experts):
+            declared[self._expert(index, "gate")] = TensorDecl((F, D))
+            declared[self._expert(index, "up")] = TensorDecl((F, D))
+            declared[self._expert(index, "down")] = TensorDecl((D, F))
+        if self.shared is not None:
+            declared.update(self.shared.tensors())
+        return declared
+
+    def bind(self, tensors, dtype, device) -> None:
+        super().bind(tensors, dtype, device)
+        self.router = tensors[self.prefix + self.names["router"]]
+        self.bias = tensors[self.prefix + self.names["router_bias"]] if self.router_bias else None
+        self.gate_up = torch.stack([torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], dim=0)
+                                    for e in range(self.experts)]).contiguous()
+        self.down = torch.stack([tensors[self._expert(e, "down")] for e in range(self.experts)]).contiguous()
+        if self.shared is not None:
+            self.shared.bind(tensors, dtype, device)
+
+    def route(self, h: torch.Tensor):
+        """(chosen [rows, top], weight [rows, top]) of the rows ``h``."""
+        logits = ops.gemm_generic(h, self.router, out_dtype=torch.float32)
+        return ops.moe_route(logits, self.bias, self.top)
+
+    def forward(self, h, residual, ctx):
+        rows = (h.tensor() if isinstance(h, LazyNorm) else h)
+        chosen, weight = self.route(rows)
+        begin, place_row, pair_place = ops.moe_arrange(chosen, self.experts)
+        places = rows.shape[0] * self.top
+        hidden = ops.grouped_gemm(rows, place_row, self.gate_up, begin, places, gated=True, out_dtype=rows.dtype)
+        outputs = ops.grouped_gemm(hidden, None, self.down, begin, places, gated=False, out_dtype=torch.float32)
+        ops.moe_combine_(residual, outputs, weight, pair_place)
+        if self.shared is not None:
+            return self.shared.forward(h, residual, ctx)
+        return None
+
+    def output(self, h, ctx) -> torch.Tensor:
+        out = torch.zeros((h.shape[0], self.hidden), dtype=torch.float32, device=h.device)
+        self.forward(h, out, ctx)
+        return out

@@ -5,9 +5,14 @@ pairs channel 2i with channel 2i + 1 instead, by the same angles (``interleaved`
 kernels which pairing the tables are for). The inverse
 frequencies are formed in float64 on the host; the per-step cos/sin tables are float32.
 ``rotary_dim = 0`` (or kind ``none``) means no position encoding at all. ``scaling_factor`` f
-(linear position scaling) divides every frequency by f: position p turns as p / f would."""
+(linear position scaling) divides every frequency by f: position p turns as p / f would.
+``wavelength_scaling`` (factor, low, high, original) stretches by wavelength instead: with l = 2 pi / f
+a frequency stays where l < original / high, becomes f / factor where l > original / low, and between the
+two is the blend (1 - s) f / factor + s f with s = (original / l - low) / (high - low)."""
 
 from __future__ import annotations
+
+import math
 
 import torch
 
@@ -31,13 +36,27 @@ class RotaryNeox(PositionEncoding):
             raise ConfigError(f"the rotation's scaling factor must be positive, found {self.scaling_factor}")
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.head_dim:
             raise ConfigError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {self.head_dim}")
+        stretch = spec.get("wavelength_scaling")
+        self.wavelength_scaling = None if stretch is None else tuple(float(number) for number in stretch)
+        if self.wavelength_scaling is not None:
+            factor, low, high, original = self.wavelength_scaling      # four numbers, or this raises
+            if not (factor > 0 and original > 0 and high > low >= 0):
+                raise ConfigError(f"the rotation's wavelength scaling needs factor > 0, original > 0 and high > low >= 0, found {stretch}")
         self._inv_freq = None
 
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
         half = self.rotary_dim // 2
         exponents = torch.arange(half, dtype=torch.float64) * 2.0 / max(self.rotary_dim, 1)
-        self._inv_freq = (self.theta ** (-exponents) / self.scaling_factor).to(device)
+        frequencies = self.theta ** (-exponents) / self.scaling_factor
+        if self.wavelength_scaling is not None:
+            factor, low, high, original = self.wavelength_scaling
+            wavelength = 2.0 * math.pi / frequencies
+            blend = (original / wavelength - low) / (high - low)
+            between = (1.0 - blend) * frequencies / factor + blend * frequencies
+            frequencies = torch.where(wavelength < original / high, frequencies,
+                                      torch.where(wavelength > original / low, frequencies / factor, between))
+        self._inv_freq = frequencies.to(device)
 
     def tables(self, ctx):
         if self.rotary_dim == 0:
