@@ -236,3 +236,77 @@ def forward(config: Dict, weights: Dict[str, np.ndarray], tokens: List[int], lay
         if layers_out is not None:
             layers_out.append(x.copy())
     return norm_around_zero(x, weights["final.norm"], eps) @ weights["head"].T * config.get("logit_scale", 1.0)
+
+
+def greedy(config: Dict, weights: Dict[str, np.ndarray], prompt: List[int], new: int) -> List[int]:
+    tokens, out = list(prompt), []
+    for _ in range(new):
+        out.append(int(np.argmax(forward(config, weights, tokens)[-1])))
+        tokens.append(out[-1])
+    return out
+
+
+# ----- tensors of a model --------------------------------------------------------------------------------
+def tensor_shapes(config: Dict, decay_rank: int = 8) -> Dict[str, Tuple[int, ...]]:
+    D, V = config["width"], config["vocab"]
+    shapes: Dict[str, Tuple[int, ...]] = {"embed": (V, D), "pos": (config["max_positions"], D), "final.norm": (D,), "head": (V, D)}
+    for index, layer in enumerate(config["layers"]):
+        base, m = f"l{index}.", layer["mixer"]
+        shapes[base + "norm1"] = (D,)
+        if layer["type"] == "wkv":
+            W = m["heads"] * m["dim"]
+            for s in "rkvgw":
+                shapes[base + "mix.mu." + s] = (D,)
+            for s in "rkvg":
+                shapes[base + "mix." + s] = (W, D)
+            rank = m.get("decay_rank", decay_rank)
+            shapes.update({base + "mix.w1": (rank, D), base + "mix.w2": (W, rank), base + "mix.w0": (W,), base + "mix.u": (m["heads"], m["dim"]),
+                           base + "mix.norm": (W,), base + "mix.o": (D, W)})
+        else:
+            H, G, d = m["heads"], m.get("kv_heads", m["heads"]), m["dim"]
+            dv = m.get("vdim", d)
+            shapes.update({base + "mix.q": (H * d, D), base + "mix.sink": (H,), base + "mix.o": (D, H * dv)})
+            if m.get("kv_from") is None:
+                shapes.update({base + "mix.k": (G * d, D), base + "mix.v": (G * dv, D)})
+        mlp = layer.get("mlp")
+        if mlp is None:
+            continue
+        units = {"": mlp["ff"]} if mlp["kind"] == "dense" else {f"e{e}.": mlp["expert"]["ff"] for e in range(mlp["router"]["experts"])}
+        if mlp["kind"] == "moe":
+            shapes.update({base + "mlp.router": (mlp["router"]["experts"], D), base + "mlp.router.b": (mlp["router"]["experts"],)})
+            if mlp.get("shared"):
+                units["shared."] = mlp["shared"]["ff"]
+        for unit, ff in units.items():
+            shapes.update({base + f"mlp.{unit}gate": (ff, D), base + f"mlp.{unit}up": (ff, D), base + f"mlp.{unit}down": (D, ff)})
+    return shapes
+
+
+def random_weights(config: Dict, seed: int, decay_rank: int = 8) -> Dict[str, np.ndarray]:
+    """Weights that make every part count: matrices keep the size of what passes through them, sinks of about one,
+    decays from barely forgetting to forgetting at once, a bonus and mixing weights of visible size."""
+    rng = np.random.default_rng(seed)
+    weights: Dict[str, np.ndarray] = {}
+    for name, shape in tensor_shapes(config, decay_rank).items():
+        leaf = name.split(".")[-1]
+        if name.endswith("norm1") or name == "final.norm":
+            value = rng.uniform(-0.3, 0.3, shape)
+        elif ".mu." in name:
+            value = rng.uniform(0.0, 1.0, shape)
+        elif leaf == "w0":
+            value = rng.uniform(-6.0, 0.5, shape)
+        elif leaf == "u":
+            value = rng.normal(0.0, 0.5, shape)
+        elif leaf == "norm":
+            value = rng.uniform(0.7, 1.3, shape)
+        elif leaf == "sink":
+            value = rng.normal(0.0, 1.5, shape)
+        elif leaf == "b":
+            value = rng.normal(0.0, 0.5, shape)
+        elif name == "pos":
+            value = rng.normal(0.0, 0.5, shape)
+        elif name == "embed":
+            value = rng.normal(0.0, 1.0, shape)
+        else:
+            value = rng.normal(0.0, 1.0, shape) / math.sqrt(shape[-1])
+        weights[name] = value
+    return weights
