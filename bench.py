@@ -114,6 +114,48 @@ def vavelorn_configs(size: dict):
     return vavelorn, koketar_configs(size)[0]
 
 
+# Dalerax (parallel layers; a wkv recurrence or windowed attention with kept first keys and a sink per head, two of
+# the attention layers on one cache entry; a dense unit or a mixture of experts with a shared unit) at two such
+# sizes, beside the engine's closest existing model: a Koketar of the same width, depth and vocabulary whose dense
+# feed-forward is as wide as the units a Dalerax token runs through (the chosen experts and the shared one).
+DALERAX_SIZES = {
+    "w1024": dict(width=1024, layers=4, vocab=32768, ff=4096, heads=8, kv_heads=2, dim=128, vdim=128, window=512, keep_first=4,
+                  rot_dims=64, r_heads=8, r_kv_heads=4, r_dim=64, r_vdim=128, conv=4, rank=32, w_heads=16, w_dim=64,
+                  experts=16, top=4, expert_ff=768, shared_ff=1024),
+    "w2048": dict(width=2048, layers=4, vocab=32768, ff=8192, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, keep_first=4,
+                  rot_dims=64, r_heads=16, r_kv_heads=8, r_dim=128, r_vdim=128, conv=4, rank=64, w_heads=32, w_dim=64,
+                  experts=32, top=4, expert_ff=1536, shared_ff=2048),
+}
+
+
+def dalerax_configs(size: dict):
+    """(Dalerax configuration, Koketar configuration of equal size)."""
+    from flyweight_amd.config import config_from_dict
+    dense = {"kind": "dense", "ff": size["ff"]}
+    moe = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"]}, "expert": {"ff": size["expert_ff"]},
+           "shared": {"ff": size["shared_ff"]}}
+    attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"],
+                 "scale": size["dim"] ** -0.5, "mask": {"size": size["window"], "keep_first": size["keep_first"]},
+                 "rot": {"dims": size["rot_dims"], "base": 1000000.0,
+                         "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}}
+    recurrence = {"heads": size["w_heads"], "dim": size["w_dim"], "decay_rank": size["rank"]}
+    kinds = [
+        {"type": "wkv", "mixer": recurrence, "mlp": dense},
+        {"type": "attention", "mixer": attention, "mlp": moe},
+        {"type": "attention", "mixer": dict(attention, kv_from=1), "mlp": moe},
+        {"type": "wkv", "mixer": recurrence, "mlp": moe},
+    ]
+    layers = []
+    for index in range(size["layers"]):
+        kind = kinds[index % 4]
+        if kind["mixer"].get("kv_from") is not None:     # the layer before it owns the keys and values
+            kind = dict(kind, mixer=dict(kind["mixer"], kv_from=index - 1))
+        layers.append(kind)
+    dalerax = config_from_dict({"architecture": "Dalerax", "vocab": size["vocab"], "width": size["width"], "max_positions": CONTEXT,
+                                "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0}, "logit_scale": 1.0, "layers": layers})
+    return dalerax, koketar_configs(size)[0]
+
+
 def kernel_times(torch, run) -> dict:
     """Entry point of the kernel library -> microseconds of GPU time per call, over one call of ``run``
     (launched kernel by kernel, every call bracketed by two events)."""
@@ -486,10 +528,10 @@ def main() -> int:
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
     parser.add_argument("--drawn", action="store_true", help="with --only decode: the requests draw their tokens "
                         "(temperature 0.8, top_k 40, top_p 0.95, min_p 0.05) instead of taking the most likely one")
-    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar", "vavelorn"), default="headline",
+    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar", "vavelorn", "dalerax"), default="headline",
                         help="headline: the LFM2-1.2B decode and prefill figures; long-context, mixed: a whole serving run; "
                              "koketar: prefill and decode of Koketar beside LFM2 at equal sizes, kernel by kernel; "
-                             "vavelorn: the same of Vavelorn beside Koketar")
+                             "vavelorn: the same of Vavelorn beside Koketar; dalerax: the same of Dalerax beside Koketar")
     parser.add_argument("--requests", type=int, help="requests of a serving workload (default: as the workload names)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -503,8 +545,12 @@ def main() -> int:
     from flyweight_amd import Model
     from flyweight_amd.config import config_from_dict
 
-    if args.workload in ("koketar", "vavelorn"):
-        if args.workload == "vavelorn":
+    if args.workload in ("koketar", "vavelorn", "dalerax"):
+        if args.workload == "dalerax":
+            record = koketar_run(torch, args, families=("dalerax", "koketar"), sizes=DALERAX_SIZES, configs_of=dalerax_configs,
+                                 title="Dalerax", beside="Dalerax beside Koketar at equal width, depth, vocabulary and feed-forward "
+                                                         "width a token runs through")
+        elif args.workload == "vavelorn":
             record = koketar_run(torch, args, families=("vavelorn", "koketar"), sizes=VAVELORN_SIZES, configs_of=vavelorn_configs,
                                  title="Vavelorn", beside="Vavelorn beside Koketar at equal width, depth, feed-forward width and vocabulary")
         else:

@@ -77,10 +77,11 @@ extern "C" int fw_moe_route(const float* logits, const float* bias, int32_t* cho
 // expert follow each other in the order of the threads, so that an expert's places hold its pairs in the
 // order (row, choice). expert_begin [experts + 1]; place_row [pairs]; pair_place [pairs].
 #define MOE_ARRANGE_THREADS 1024
+#define MOE_ARRANGE_STAGED 10240        // pairs whose experts are kept in LDS (40 KB)
 __global__ __launch_bounds__(MOE_ARRANGE_THREADS) void moe_arrange_kernel(const int32_t* __restrict__ chosen, int32_t* __restrict__ expert_begin,
                                                                           int32_t* __restrict__ place_row, int32_t* __restrict__ pair_place,
-                                                                          int pairs, int experts, int top) {
-    extern __shared__ int32_t counts[];         // [experts + 1] begins, then [threads-in-use][experts] is too much: runs are walked twice instead
+                                                                          int pairs, int experts, int top, int staged) {
+    extern __shared__ int32_t counts[];         // [experts + 1] begins, then the experts of the first `staged` pairs
     const int tid = threadIdx.x;
     for (int e = tid; e <= experts; e += MOE_ARRANGE_THREADS) counts[e] = 0;
     __syncthreads();
@@ -98,15 +99,20 @@ __global__ __launch_bounds__(MOE_ARRANGE_THREADS) void moe_arrange_kernel(const 
     __syncthreads();
     for (int e = tid; e <= experts; e += MOE_ARRANGE_THREADS) expert_begin[e] = counts[e];
     // Places in order: a wave per expert at a time walks all pairs in runs of 64 and numbers those of its
-    // expert by a prefix count over the lanes (ballot), so the order is that of the pairs.
+    // expert by a prefix count over the lanes (ballot), so the order is that of the pairs. The walk is one
+    // dependent read after the other: the pairs' experts are first copied behind the counters in LDS where
+    // they fit (staged > 0), and read from there.
+    int32_t* mine = counts + experts + 1;
+    for (int i = tid; i < staged; i += MOE_ARRANGE_THREADS) mine[i] = chosen[i];
+    __syncthreads();
     const int lane = tid & 63, wave = tid >> 6, waves = MOE_ARRANGE_THREADS / 64;
     for (int e = wave; e < experts; e += waves) {
         int next = counts[e];
-        const int end = e + 1 <= experts ? counts[e + 1] : pairs;
+        const int end = counts[e + 1];
         if (next == end) continue;
-        for (int i0 = 0; i0 < pairs; i0 += 64) {
+        for (int i0 = 0; i0 < pairs && next < end; i0 += 64) {
             const int i = i0 + lane;
-            const bool is_mine = i < pairs && chosen[i] == e;
+            const bool is_mine = i < pairs && (i < staged ? mine[i] : chosen[i]) == e;
             const unsigned long long votes = __ballot(is_mine);
             if (is_mine) {
                 const int place = next + __popcll(votes & ((1ull << lane) - 1ull));
@@ -122,8 +128,10 @@ extern "C" int fw_moe_arrange(const int32_t* chosen, int32_t* expert_begin, int3
                               int top, void* stream) {
     FW_REQUIRE(rows >= 0 && experts >= 1 && experts <= MOE_MAX_EXPERTS && top >= 1, "moe_arrange: bad sizes rows=%d experts=%d top=%d", rows, experts, top);
     FW_REQUIRE((long long)rows * top < (1ll << 30), "moe_arrange: too many pairs");
-    moe_arrange_kernel<<<1, MOE_ARRANGE_THREADS, (experts + 1) * sizeof(int32_t), (hipStream_t)stream>>>(chosen, expert_begin, place_row, pair_place,
-                                                                                                        rows * top, experts, top);
+    const int pairs = rows * top;
+    const int staged = pairs <= MOE_ARRANGE_STAGED ? pairs : MOE_ARRANGE_STAGED;
+    moe_arrange_kernel<<<1, MOE_ARRANGE_THREADS, (experts + 1 + staged) * sizeof(int32_t), (hipStream_t)stream>>>(
+        chosen, expert_begin, place_row, pair_place, pairs, experts, top, staged);
     FW_LAUNCH_CHECK("moe_arrange");
     return 0;
 }
@@ -221,15 +229,272 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const TA* __restrict_
     }
 }
 
+// ---- the grouped product on the matrix cores -----------------------------------------------------------
+// bfloat16 operands, float32 accumulation (v_mfma_f32_32x32x16_bf16). A tile of places belongs to one
+// expert; both operands are k-contiguous, a slab of 64 k of each is copied per iteration: global ->
+// registers (two slabs ahead of the one multiplied) -> LDS (one ahead), two LDS buffers, one barrier an
+// iteration, LDS rows padded to 144 bytes. Two shapes of tile:
+//   BIG     128 places x 128 rows of W; four waves as 2 x 2, each 64 x 64. For steps in which an expert
+//           has hundreds of places (prompts): the product is bound by the matrix cores.
+//   small    32 places x (128 NJ) rows of W; four waves side by side, each 32 x (32 NJ). For steps of
+//           few places an expert (decoding): the product is bound by how fast the experts' weights stream,
+//           and every workgroup streams rows of W that no other reads.
+// GATED: W is [2 N][K], gate rows then up rows; a tile takes as many gate rows as up rows of the same
+// features, a wave holds gate and up of one element in one lane and stores silu(gate) * up.
+// Which tile a workgroup has: tiles are numbered over all experts one after the other (an expert with n
+// places has ceil(n / rows) of them); a wave finds its expert by a prefix sum of 64 experts' tile counts
+// at a time. The grid holds as many tiles as there can be at most; a workgroup beyond the last leaves.
+// A place's sum over k is formed in one order whatever the tile's shape and whoever shares the tile.
+typedef __attribute__((ext_vector_type(8))) __bf16 gg_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float gg_f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t gg_u32x4;
+#define GGM_TK 64
+#define GGM_ROW_BYTES 144
+#define GGM_GROUP 8
+
+__device__ __forceinline__ float gg_silu(float g) {
+    if (g >= 0.0f) return g / (1.0f + __expf(-g));
+    const float e = __expf(g);
+    return g * e / (1.0f + e);
+}
+
+template <bool GATED, bool BIG, int NJ, typename TO>
+__global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(
+    const uint16_t* __restrict__ a, const int32_t* __restrict__ place_row, const uint16_t* __restrict__ w,
+    const int32_t* __restrict__ expert_begin, TO* __restrict__ out, int experts, int N, int K, int tiles_m, int tiles_n, int per_xcd) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    constexpr int TMR = BIG ? 128 : 32;                 // places of a tile
+    constexpr int WAVES_M = BIG ? 2 : 1, WAVES_N = 4 / WAVES_M;
+    constexpr int NI = TMR / (32 * WAVES_M);
+    constexpr int BN = WAVES_N * NJ * 32;               // rows of W of a tile
+    constexpr int A_CHUNKS = TMR / 32, W_CHUNKS = BN / 32;
+    constexpr int A_SLAB = TMR * GGM_ROW_BYTES, W_SLAB = BN * GGM_ROW_BYTES;
+    static_assert(!GATED || NJ == 2, "the gated tile holds gate and up side by side");
+    const int total = tiles_m * tiles_n;
+    const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= total) return;
+    const int width = GGM_GROUP * tiles_n;
+    const int group = logical / width;
+    const int first_m = group * GGM_GROUP;
+    const int group_size = tiles_m - first_m < GGM_GROUP ? tiles_m - first_m : GGM_GROUP;
+    const int pid_m = first_m + (logical % width) % group_size;
+    const int pid_n = (logical % width) / group_size;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+    // the expert of tile pid_m, and the tile's place among that expert's
+    int expert = -1, tile_in_expert = 0;
+    {
+        int before = 0;
+        for (int e0 = 0; e0 < experts; e0 += 64) {
+            const int e = e0 + lane;
+            const int mine = e < experts ? (expert_begin[e + 1] - expert_begin[e] + TMR - 1) / TMR : 0;
+            int upto = mine;
+#pragma unroll
+            for (int offset = 1; offset < 64; offset <<= 1) {
+                const int other = __shfl_up(upto, offset, 64);
+                if (lane >= offset) upto += other;
+            }
+            const unsigned long long holds = __ballot(pid_m < before + upto);
+            if (holds) {
+                const int at = __ffsll((long long)holds) - 1;
+                expert = e0 + at;
+                tile_in_expert = pid_m - (before + __shfl(upto, at, 64) - __shfl(mine, at, 64));
+                break;
+            }
+            before += __shfl(upto, 63, 64);
+        }
+    }
+    if (expert < 0) return;
+    const int first = expert_begin[expert] + tile_in_expert * TMR, end = expert_begin[expert + 1];
+    const int features = GATED ? BN / 2 : BN;
+    const int n0 = pid_n * features;
+    const int wm = BIG ? wave >> 1 : 0, wn = BIG ? wave & 1 : wave;
+    const uint16_t* we = w + (size_t)expert * (GATED ? 2 : 1) * N * K;
+
+    const uint16_t* a_src[A_CHUNKS];
+    const uint16_t* w_src[W_CHUNKS];
+    int a_at[A_CHUNKS], w_at[W_CHUNKS];
+    const int kc = (tid & 7) * 8;
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+        const int row = (tid >> 3) + 32 * i;
+        int place = first + row;
+        place = place < end ? place : end - 1;          // places past the expert's last are computed and dropped
+        const int from = place_row ? place_row[place] : place;
+        a_src[i] = a + (size_t)from * K;
+        a_at[i] = row * GGM_ROW_BYTES + (tid & 7) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < W_CHUNKS; ++i) {
+        const int row = (tid >> 3) + 32 * i;
+        int wr;
+        if (GATED) {
+            wr = row < BN / 2 ? n0 + row : n0 + row - BN / 2;
+            wr = wr < N ? wr : N - 1;
+            if (row >= BN / 2) wr += N;
+        } else {
+            wr = n0 + row;
+            wr = wr < N ? wr : N - 1;
+        }
+        w_src[i] = we + (size_t)wr * K;
+        w_at[i] = row * GGM_ROW_BYTES + (tid & 7) * 16;
+    }
+
+    gg_f32x16 acc[NI][NJ];
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    gg_u32x4 ra0[A_CHUNKS], rw0[W_CHUNKS], ra1[A_CHUNKS], rw1[W_CHUNKS];
+    const gg_u32x4 zero = {0u, 0u, 0u, 0u};
+    // Every load is issued unconditionally (past the end of K from column 0) and nothing touches the value
+    // until it moves to LDS, so that the loads of two slabs stay in flight while a third is multiplied.
+    auto fetch = [&](gg_u32x4 (&ra)[A_CHUNKS], gg_u32x4 (&rw)[W_CHUNKS], int k0) {
+        const int from = k0 + kc < K ? k0 + kc : 0;     // K is a multiple of 8: columns 0..7 always exist
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) ra[i] = *reinterpret_cast<const gg_u32x4*>(a_src[i] + from);
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) rw[i] = *reinterpret_cast<const gg_u32x4*>(w_src[i] + from);
+    };
+    auto stash = [&](const gg_u32x4 (&ra)[A_CHUNKS], const gg_u32x4 (&rw)[W_CHUNKS], int buffer, int k0) {
+        unsigned char* base = lds + buffer * (A_SLAB + W_SLAB);
+        const bool ok = k0 + kc < K;                    // a past the end of K is zero; W may then be anything finite
+#pragma unroll
+        for (int i = 0; i < A_CHUNKS; ++i) *reinterpret_cast<gg_u32x4*>(base + a_at[i]) = ok ? ra[i] : zero;
+#pragma unroll
+        for (int i = 0; i < W_CHUNKS; ++i) *reinterpret_cast<gg_u32x4*>(base + A_SLAB + w_at[i]) = ok ? rw[i] : zero;
+    };
+    const int a_row0 = wm * 32 * NI + (lane & 31);
+    int b_row[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+        b_row[j] = GATED ? j * (BN / 2) + wn * 32 + (lane & 31) : wn * (32 * NJ) + j * 32 + (lane & 31);
+    const int k_lane = (lane >> 5) * 16;                // byte offset of this lane's 8 k within a k16 step
+    auto multiply = [&](int buffer) {
+        const unsigned char* sa = lds + buffer * (A_SLAB + W_SLAB);
+        const unsigned char* sb = sa + A_SLAB;
+#pragma unroll
+        for (int k16 = 0; k16 < GGM_TK / 16; ++k16) {
+            gg_bf16x8 fa[NI], fb[NJ];
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+                fa[i] = *reinterpret_cast<const gg_bf16x8*>(sa + (a_row0 + 32 * i) * GGM_ROW_BYTES + k16 * 32 + k_lane);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                fb[j] = *reinterpret_cast<const gg_bf16x8*>(sb + b_row[j] * GGM_ROW_BYTES + k16 * 32 + k_lane);
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+                for (int j = 0; j < NJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    // slab s travels: global -> register set s % 2 (requested while slab s - 2 is multiplied) -> LDS buffer
+    // s % 2 (stored while slab s - 1 is multiplied) -> multiplied
+    const int steps = (K + GGM_TK - 1) / GGM_TK;
+    int step = 0;
+    fetch(ra0, rw0, 0);
+    fetch(ra1, rw1, GGM_TK);                            // past the end: dropped when stored
+    stash(ra0, rw0, 0, 0);
+    fw_lds_barrier();
+    while (step + 3 < steps) {
+        fetch(ra0, rw0, (step + 2) * GGM_TK);
+        __builtin_amdgcn_sched_barrier(0);              // keep the requests ahead of the work they overlap
+        multiply(0);
+        stash(ra1, rw1, 1, (step + 1) * GGM_TK);
+        fw_lds_barrier();
+        fetch(ra1, rw1, (step + 3) * GGM_TK);
+        __builtin_amdgcn_sched_barrier(0);
+        multiply(1);
+        stash(ra0, rw0, 0, (step + 2) * GGM_TK);
+        fw_lds_barrier();
+        step += 2;
+    }
+    // at most three slabs are left: slab `step` is in buffer 0, slab step + 1 in set 1
+    if (step + 2 < steps) fetch(ra0, rw0, (step + 2) * GGM_TK);
+    multiply(0);
+    if (step + 1 < steps) {
+        stash(ra1, rw1, 1, (step + 1) * GGM_TK);
+        fw_lds_barrier();
+        multiply(1);
+        if (step + 2 < steps) {
+            stash(ra0, rw0, 0, (step + 2) * GGM_TK);
+            fw_lds_barrier();
+            multiply(0);
+        }
+    }
+    fw_mfma_drain();     // the branches below lead to code that reads the accumulators
+
+    // D layout of the 32x32 product: lane holds column lane % 32; register r is row 8 * (r / 4) + 4 * (lane / 32) + r % 4
+    const int col = lane & 31, row_base = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int place = first + wm * 32 * NI + i * 32 + 8 * (r >> 2) + row_base + (r & 3);
+            if (place >= end) continue;
+            if (GATED) {
+                const int n = n0 + wn * 32 + col;
+                if (n < N) store_from_float(out, (size_t)place * N + n, gg_silu(acc[i][0][r]) * acc[i][NJ - 1][r]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    const int n = n0 + wn * (32 * NJ) + j * 32 + col;
+                    if (n < N) store_from_float(out, (size_t)place * N + n, acc[i][j][r]);
+                }
+            }
+        }
+}
+
+template <bool GATED, bool BIG, int NJ, typename TO>
+static int grouped_mfma_launch(const void* a, const int32_t* place_row, const void* w, const int32_t* expert_begin, void* out, int places,
+                               int experts, int N, int K, hipStream_t stream) {
+    constexpr int TMR = BIG ? 128 : 32;
+    constexpr int BN = (BIG ? 2 : 4) * NJ * 32;
+    const int features = GATED ? BN / 2 : BN;
+    const long long tiles_m = (long long)places / TMR + (experts < places ? experts : places);    // at most
+    const long long tiles_n = fw_ceil_div(N, features);
+    FW_REQUIRE(tiles_m * tiles_n < (1ll << 30), "grouped_gemm: too many tiles");
+    const int per_xcd = (int)fw_ceil_div(tiles_m * tiles_n, 8);
+    const int lds_bytes = 2 * (TMR + BN) * GGM_ROW_BYTES;
+    static bool configured = false;     // per instantiation
+    if (!configured) {
+        hipError_t status = hipFuncSetAttribute((const void*)grouped_gemm_mfma_kernel<GATED, BIG, NJ, TO>,
+                                                hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        FW_REQUIRE(status == hipSuccess, "grouped_gemm: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(status));
+        configured = true;
+    }
+    grouped_gemm_mfma_kernel<GATED, BIG, NJ, TO><<<per_xcd * 8, 256, lds_bytes, stream>>>(
+        (const uint16_t*)a, place_row, (const uint16_t*)w, expert_begin, (TO*)out, experts, N, K, (int)tiles_m, (int)tiles_n, per_xcd);
+    return 0;
+}
+
 extern "C" int fw_grouped_gemm(const void* a, int a_dtype, const int32_t* place_row, const void* w, int w_dtype,
                                const int32_t* expert_begin, void* out, int out_dtype, int gated, int places, int experts, int N, int K,
                                void* stream) {
     FW_REQUIRE(places >= 0 && experts >= 1 && N > 0 && K > 0, "grouped_gemm: bad sizes places=%d experts=%d N=%d K=%d", places, experts, N, K);
     if (places == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    // bfloat16 operands go to the matrix cores: tiles of 128 places where experts have many, of 32 where few
+    if (a_dtype == FW_BF16 && w_dtype == FW_BF16 && K % 8 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+        (out_dtype == FW_F32 || (out_dtype == FW_BF16 && gated))) {
+        const bool big = (long long)places >= 48ll * experts;
+        int status;
+        if (gated) status = big ? grouped_mfma_launch<true, true, 2, bf16_t>(a, place_row, w, expert_begin, out, places, experts, N, K, s)
+                                : grouped_mfma_launch<true, false, 2, bf16_t>(a, place_row, w, expert_begin, out, places, experts, N, K, s);
+        else status = big ? grouped_mfma_launch<false, true, 2, float>(a, place_row, w, expert_begin, out, places, experts, N, K, s)
+                          : grouped_mfma_launch<false, false, 1, float>(a, place_row, w, expert_begin, out, places, experts, N, K, s);
+        if (status != 0) return status;
+        FW_LAUNCH_CHECK("grouped_gemm");
+        return 0;
+    }
     const long long tiles = (long long)places / GG_ROWS + experts;      // at most: every expert may end in a tile that is not full
     FW_REQUIRE(tiles < (1ll << 31) && (N + GG_COLS - 1) / GG_COLS <= 65535, "grouped_gemm: grid too large");
     dim3 grid((unsigned)tiles, (N + GG_COLS - 1) / GG_COLS);
-    hipStream_t s = (hipStream_t)stream;
 #define FW_GG_LAUNCH(TA, TW, TO)                                                                                                   \
     {                                                                                                                              \
         if (gated) grouped_gemm_kernel<TA, TW, TO, true><<<grid, 256, 0, s>>>((const TA*)a, place_row, (const TW*)w, expert_begin, \

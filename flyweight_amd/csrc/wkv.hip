@@ -90,85 +90,162 @@ extern "C" int fw_tanh_rows(const float* x, void* out, int out_dtype, long long 
 }
 
 // ---- the recurrence ------------------------------------------------------------------------------
-// A wave per (segment, head, 16 value channels). Lane = 16 p + c: value channel c of the tile, key
-// channels p, p + 4, p + 8, ... (KPT of them: a quarter of the head's, interleaved so that the four lanes
-// of a column read neighbouring words of LDS). A column's sum over key channels is each lane's own sum and
-// then the four lanes' (two row swaps). Tokens come in chunks of WKV_CHUNK: the wave stages a chunk's r, k
-// and decays in LDS (the decay's two exponentials are taken here, once per chunk and key channel), forms
-// each token's bonus sum r . (u k), and then walks the chunk token by token. The state is read at the
-// segment's start and written at its end. Columns of S never meet, so the result does not depend on how
-// the work is cut; tokens are walked in order whatever the segments, so it does not depend on the cut of
-// the sequence either.
-#define WKV_CHUNK 16
-template <int KPT>
-__global__ __launch_bounds__(64) void wkv_recurrence_kernel(
+// Workgroup (segment, head, block of 16 value channels); thread = 16 * column + part: a column of S is
+// shared out over the 16 lanes of a row of the wave, RPT key channels each (part, part + 16, ...: the
+// sixteen lanes read sixteen neighbouring floats of r, k and the decay from LDS; channels from dim on hold
+// zeros), so that a head is spread over many compute units: the walk along the tokens is one dependent
+// chain per column (a single multiply-add per key channel and token), and only its width can be bought.
+// Tokens come in chunks of WKV_CHUNK (16, fewer for wide heads, whose tokens are larger). A chunk's r, k, a and its block's 16 values travel from global
+// memory into registers while the chunk before is walked; on their way into LDS the decay's two
+// exponentials are taken, once per chunk and key channel. A column's sums over key channels (the read-out
+// S^T r and the bonus r . (u k), which every column forms for itself) are each thread's own sum and then
+// the sixteen lanes', inside the vector unit. The state is read at the segment's start and written at its
+// end. Columns of S never meet and the lanes' sums have one fixed order, so the result depends neither on
+// how the work is cut nor, tokens being walked in order whatever the segments, on the cut of the sequence.
+#define WKV_LANES 16
+#define WKV_COLUMNS (256 / WKV_LANES)
+template <int CTRL>
+__device__ __forceinline__ float wkv_dpp(float x) {
+    return __uint_as_float((uint32_t)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(x), CTRL, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float wkv_row_sum(float x) {
+    x += wkv_dpp<0xB1>(x);          // quad_perm [1, 0, 3, 2]
+    x += wkv_dpp<0x4E>(x);          // quad_perm [2, 3, 0, 1]
+    x += wkv_dpp<0x141>(x);         // row_half_mirror
+    x += wkv_dpp<0x140>(x);         // row_mirror
+    return x;
+}
+
+template <int RPT, int WKV_CHUNK>
+__global__ __launch_bounds__(256) void wkv_recurrence_kernel(
     const float* __restrict__ r, const float* __restrict__ k, const float* __restrict__ v, int rkv_stride,
     const float* __restrict__ a, int a_stride, const float* __restrict__ w0, const float* __restrict__ u, float* __restrict__ state,
     float* __restrict__ out, const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot, int heads, int dim) {
-    extern __shared__ float lds[];
-    const int padded = KPT * 4;                     // key channels as the lanes hold them
-    float* rs = lds;                                // [WKV_CHUNK][padded]
-    float* ks = rs + WKV_CHUNK * padded;
-    float* ws = ks + WKV_CHUNK * padded;
-    float* bonus = ws + WKV_CHUNK * padded;         // [WKV_CHUNK]
-    const int seg = blockIdx.x, head = blockIdx.y, tile = blockIdx.z;
-    const int lane = threadIdx.x, c = lane & 15, p = lane >> 4;
-    const int column = tile * 16 + c;
-    const bool column_there = column < dim;
-    const int row0 = seg_row0[seg], row_end = seg_row0[seg + 1];
-    float* S = state + ((size_t)seg_slot[seg] * heads + head) * dim * dim;
-    float s[KPT];
-#pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-        const int key = 4 * i + p;
-        s[i] = (key < dim && column_there) ? S[(size_t)key * dim + column] : 0.0f;
-    }
+    constexpr int DP = WKV_LANES * RPT;                 // key channels as the lanes hold them
+    constexpr int TOKEN = 3 * DP + WKV_COLUMNS;         // a staged token: r, k, decay, the block's values
+    constexpr int PIECES = (WKV_CHUNK * TOKEN + 255) / 256;
+    __shared__ float staged[WKV_CHUNK * TOKEN];
+    __shared__ float results[WKV_CHUNK * WKV_COLUMNS];
+    __shared__ float w0s[DP];                           // the decay's offsets of this head
+    static_assert(WKV_CHUNK * WKV_COLUMNS <= 256, "a chunk's read-outs are at most one per thread");
+    const int seg = blockIdx.x, head = blockIdx.y, block = blockIdx.z;
+    const int local = threadIdx.x / WKV_LANES, part = threadIdx.x % WKV_LANES;
+    const int column = block * WKV_COLUMNS + local;
+    const bool live = column < dim;
+    const int first = seg_row0[seg], count = seg_row0[seg + 1] - first;
     const size_t head_at = (size_t)head * dim;
-    for (int chunk0 = row0; chunk0 < row_end; chunk0 += WKV_CHUNK) {
-        const int count = row_end - chunk0 < WKV_CHUNK ? row_end - chunk0 : WKV_CHUNK;
-        for (int item = lane; item < count * padded; item += 64) {
-            const int t = item / padded, key = item % padded;
-            const size_t row = chunk0 + t;
-            float rv = 0.0f, kv = 0.0f, wv = 0.0f;
-            if (key < dim) {
-                rv = r[row * rkv_stride + head_at + key];
-                kv = k[row * rkv_stride + head_at + key];
-                wv = expf(-expf(a[row * a_stride + head_at + key] + w0[head_at + key]));
-            }
-            rs[item] = rv;
-            ks[item] = kv;
-            ws[item] = wv;
-        }
-        fw_lds_barrier();
-        for (int t = 0; t < count; ++t) {
-            float part = 0.0f;
-            for (int key = lane; key < dim; key += 64) part = fmaf(rs[t * padded + key] * u[head_at + key], ks[t * padded + key], part);
-            part = wave_sum(part);
-            if (lane == 0) bonus[t] = part;
-        }
-        fw_lds_barrier();
-        for (int t = 0; t < count; ++t) {
-            const size_t row = chunk0 + t;
-            const float value = column_there ? v[row * rkv_stride + head_at + column] : 0.0f;
-            const float* rt = rs + t * padded;
-            const float* kt = ks + t * padded;
-            const float* wt = ws + t * padded;
-            float sum = 0.0f;
+    // this thread's pieces of every chunk, one float each: token of the chunk, array (0 r, 1 k, 2 a, 3 v) and channel
+    const int per_token = 3 * dim + WKV_COLUMNS;
+    int piece[PIECES];
 #pragma unroll
-            for (int i = 0; i < KPT; ++i) {
-                const int key = 4 * i + p;
-                sum = fmaf(rt[key], s[i], sum);
-                s[i] = fmaf(wt[key], s[i], kt[key] * value);
-            }
-            sum = fw_quad_sum(sum);
-            if (p == 0 && column_there) out[row * (size_t)heads * dim + head_at + column] = fmaf(bonus[t], value, sum);
+    for (int i = 0; i < PIECES; ++i) {
+        const int item = threadIdx.x + 256 * i;
+        const int token = item / per_token, f = item % per_token;
+        int which = f / dim, channel = f % dim;
+        if (which >= 3) {
+            which = 3;
+            channel = f - 3 * dim;
+            if (block * WKV_COLUMNS + channel >= dim) which = 4;     // a column past the head: no such value
         }
-        fw_lds_barrier();       // the next chunk overwrites what this walk has read
+        piece[i] = token < WKV_CHUNK ? (token << 16) | (which << 12) | channel : -1;
     }
+    const int staged_tokens = count < WKV_CHUNK ? count : WKV_CHUNK;        // a decode step stages one token
+    for (int i = threadIdx.x; i < staged_tokens * TOKEN; i += 256) staged[i] = 0.0f;
+    for (int i = threadIdx.x; i < DP; i += 256) w0s[i] = i < dim ? w0[head_at + i] : 0.0f;
+    float held[PIECES];
+    // Loads are unconditional (a piece past the chunk's end is read from a valid place again and never used):
+    // behind a branch the compiler would wait for each load at once, and the next chunk would not travel while
+    // this one is walked.
+    auto ask = [&](int base) {
+        const int last = (count - base < WKV_CHUNK ? count - base : WKV_CHUNK) - 1;
 #pragma unroll
-    for (int i = 0; i < KPT; ++i) {
-        const int key = 4 * i + p;
-        if (key < dim && column_there) S[(size_t)key * dim + column] = s[i];
+        for (int i = 0; i < PIECES; ++i) {
+            const int code = piece[i] < 0 ? 0 : piece[i];
+            int token = code >> 16;
+            token = token < last ? token : last;
+            const int which = (code >> 12) & 7, channel = code & 0xfff;
+            const size_t row = (size_t)(first + base + token);
+            const float* from = which == 0 ? r + row * rkv_stride + head_at + channel
+                              : which == 1 ? k + row * rkv_stride + head_at + channel
+                              : which == 2 ? a + row * a_stride + head_at + channel
+                              : which == 3 ? v + row * rkv_stride + head_at + block * WKV_COLUMNS + channel
+                                           : r + row * rkv_stride + head_at;
+            held[i] = *from;
+        }
+    };
+    auto put = [&](int base) {
+        const int tokens = count - base < WKV_CHUNK ? count - base : WKV_CHUNK;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int code = piece[i];
+            if (code < 0 || (code >> 16) >= tokens) continue;
+            const int token = code >> 16, which = (code >> 12) & 7, channel = code & 0xfff;
+            if (which == 4) continue;
+            float value = held[i];
+            if (which == 2) value = expf(-expf(value + w0s[channel]));
+            staged[token * TOKEN + (which < 3 ? which * DP + channel : 3 * DP + channel)] = value;
+        }
+    };
+    ask(0);
+    float* mine = state + ((size_t)seg_slot[seg] * heads + head) * dim * dim + (live ? column : 0);
+    float S[RPT], bonus[RPT];
+#pragma unroll
+    for (int t = 0; t < RPT; ++t) {
+        const int key = t * WKV_LANES + part;
+        S[t] = (live && key < dim) ? mine[(size_t)key * dim] : 0.0f;
+        bonus[t] = key < dim ? u[head_at + key] : 0.0f;
+    }
+    __syncthreads();        // the zeros and the offsets are in place
+    put(0);
+    __syncthreads();
+    for (int base = 0; base < count; base += WKV_CHUNK) {
+        const int tokens = count - base < WKV_CHUNK ? count - base : WKV_CHUNK;
+        const bool more = base + WKV_CHUNK < count;
+        if (more) ask(base + WKV_CHUNK);
+        // a token's operands are read from LDS while the token before it is worked on
+        float r_next[RPT], k_next[RPT], w_next[RPT], v_next;
+        auto fetch = [&](int token) {
+            const float* t0 = staged + token * TOKEN;
+#pragma unroll
+            for (int t = 0; t < RPT; ++t) {
+                r_next[t] = t0[t * WKV_LANES + part];
+                k_next[t] = t0[DP + t * WKV_LANES + part];
+                w_next[t] = t0[2 * DP + t * WKV_LANES + part];
+            }
+            v_next = t0[3 * DP + local];
+        };
+        fetch(0);
+        for (int token = 0; token < tokens; ++token) {
+            const float value = v_next;
+            float read = 0.0f, ruk = 0.0f;
+#pragma unroll
+            for (int t = 0; t < RPT; ++t) {
+                read = fmaf(r_next[t], S[t], read);
+                ruk = fmaf(r_next[t] * bonus[t], k_next[t], ruk);
+                S[t] = fmaf(w_next[t], S[t], k_next[t] * value);
+            }
+            fetch(token + 1 < staged_tokens ? token + 1 : token);       // (behind the chunk's last token: read again, not used)
+            read = wkv_row_sum(read);
+            ruk = wkv_row_sum(ruk);
+            if (part == 0) results[token * WKV_COLUMNS + local] = fmaf(ruk, value, read);
+        }
+        // (barriers that order LDS traffic only: the next chunk's loads stay in flight across them)
+        fw_lds_barrier();
+        // the chunk's read-outs leave together: a token's 16 columns side by side
+        {
+            const int token = threadIdx.x / WKV_COLUMNS, c = threadIdx.x % WKV_COLUMNS;
+            if (token < tokens && block * WKV_COLUMNS + c < dim)
+                out[((size_t)first + base + token) * heads * dim + head_at + block * WKV_COLUMNS + c] = results[threadIdx.x];
+        }
+        if (more) put(base + WKV_CHUNK);
+        fw_lds_barrier();
+    }
+    if (live) {
+#pragma unroll
+        for (int t = 0; t < RPT; ++t) {
+            const int key = t * WKV_LANES + part;
+            if (key < dim) mine[(size_t)key * dim] = S[t];
+        }
     }
 }
 
@@ -179,25 +256,15 @@ extern "C" int fw_wkv_recurrence(const float* r, const float* k, const float* v,
     FW_REQUIRE(dim >= 1 && dim <= 256, "wkv_recurrence: a head of %d channels (1..256)", dim);
     FW_REQUIRE(rkv_stride >= heads * dim && a_stride >= heads * dim, "wkv_recurrence: rows of %d / %d values do not hold %d heads of %d", rkv_stride, a_stride, heads, dim);
     if (rows == 0 || segments == 0) return 0;
-    dim3 grid(segments, heads, (dim + 15) / 16);
+    dim3 grid(segments, heads, (dim + WKV_COLUMNS - 1) / WKV_COLUMNS);
     hipStream_t s = (hipStream_t)stream;
-#define FW_WKV_LAUNCH(KPT)                                                                                                     \
-    {                                                                                                                          \
-        const int lds_bytes = (3 * WKV_CHUNK * KPT * 4 + WKV_CHUNK) * 4;                                                       \
-        static int configured = 0;                                                                                             \
-        if (lds_bytes > 48 * 1024 && lds_bytes > configured) {                                                                 \
-            hipError_t status = hipFuncSetAttribute((const void*)wkv_recurrence_kernel<KPT>,                                   \
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);                    \
-            FW_REQUIRE(status == hipSuccess, "wkv_recurrence: cannot reserve %d bytes of LDS", lds_bytes);                     \
-            configured = lds_bytes;                                                                                            \
-        }                                                                                                                      \
-        wkv_recurrence_kernel<KPT><<<grid, 64, lds_bytes, s>>>(r, k, v, rkv_stride, a, a_stride, w0, u, state, out, seg_row0,  \
-                                                               seg_slot, heads, dim);                                         \
-    }
-    if (dim <= 32) FW_WKV_LAUNCH(8)
-    else if (dim <= 64) FW_WKV_LAUNCH(16)
-    else if (dim <= 128) FW_WKV_LAUNCH(32)
-    else FW_WKV_LAUNCH(64)
+#define FW_WKV_LAUNCH(RPT, CHUNK) \
+    wkv_recurrence_kernel<RPT, CHUNK><<<grid, 256, 0, s>>>(r, k, v, rkv_stride, a, a_stride, w0, u, state, out, seg_row0, seg_slot, heads, dim)
+    if (dim <= 16) FW_WKV_LAUNCH(1, 16);
+    else if (dim <= 32) FW_WKV_LAUNCH(2, 16);
+    else if (dim <= 64) FW_WKV_LAUNCH(4, 16);
+    else if (dim <= 128) FW_WKV_LAUNCH(8, 8);
+    else FW_WKV_LAUNCH(16, 4);
 #undef FW_WKV_LAUNCH
     FW_LAUNCH_CHECK("wkv_recurrence");
     return 0;

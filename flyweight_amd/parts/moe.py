@@ -19,6 +19,7 @@ from ..config.spec import ConfigError, PartSpec
 from ..kernels import ops
 from ..weights.loader import TensorDecl
 from .base import FeedForward, build_part, register_feed_forward
+from .linear import Linear
 from .norm import LazyNorm
 
 _DEFAULT_NAMES = {"router": "router", "router_bias": "router.b", "expert": "e{index}.", "gate": "gate", "up": "up", "down": "down",
@@ -56,8 +57,8 @@ class MoeSwiGLU(FeedForward):
 
     def tensors(self) -> Dict[str, TensorDecl]:
         D, F = self.hidden, self.intermediate
-        # the router decides in float32: its weights are widened once, when they are loaded
-        declared = {self.prefix + self.names["router"]: TensorDecl((self.experts, D), "vector", "matrix")}
+        # the router's product sums in float32 (its operands' products are exact there) and leaves float32 logits
+        declared = {self.prefix + self.names["router"]: TensorDecl((self.experts, D))}
         if self.router_bias:
             declared[self.prefix + self.names["router_bias"]] = TensorDecl((self.experts,), "vector", "bias")
         for index in range(self.experts):
@@ -70,7 +71,7 @@ class MoeSwiGLU(FeedForward):
 
     def bind(self, tensors, dtype, device) -> None:
         super().bind(tensors, dtype, device)
-        self.router = tensors[self.prefix + self.names["router"]]
+        self.router = Linear(tensors[self.prefix + self.names["router"]])
         self.bias = tensors[self.prefix + self.names["router_bias"]] if self.router_bias else None
         self.gate_up = torch.stack([torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], dim=0)
                                     for e in range(self.experts)]).contiguous()
@@ -80,7 +81,7 @@ class MoeSwiGLU(FeedForward):
 
     def route(self, h: torch.Tensor):
         """(chosen [rows, top], weight [rows, top]) of the rows ``h``."""
-        logits = ops.gemm_generic(h, self.router, out_dtype=torch.float32)
+        logits = self.router.forward(h, out_dtype=torch.float32)
         return ops.moe_route(logits, self.bias, self.top)
 
     def forward(self, h, residual, ctx):
