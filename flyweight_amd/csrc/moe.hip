@@ -241,16 +241,15 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const TA* __restrict_
 //           and every workgroup streams rows of W that no other reads.
 // GATED: W is [2 N][K], gate rows then up rows; a tile takes as many gate rows as up rows of the same
 // features, a wave holds gate and up of one element in one lane and stores silu(gate) * up.
-// Which tile a workgroup has: tiles are numbered over all experts one after the other (an expert with n
-// places has ceil(n / rows) of them); a wave finds its expert by a prefix sum of 64 experts' tile counts
-// at a time. The grid holds as many tiles as there can be at most; a workgroup beyond the last leaves.
+// Which tile a workgroup has: an expert with n places has ceil(n / rows) tiles of places, each times the
+// tiles of features; a wave finds its expert by a prefix sum of 64 experts' tile counts at a time. The grid
+// holds as many tiles as there can be at most; a workgroup beyond the last leaves.
 // A place's sum over k is formed in one order whatever the tile's shape and whoever shares the tile.
 typedef __attribute__((ext_vector_type(8))) __bf16 gg_bf16x8;
 typedef __attribute__((ext_vector_type(16))) float gg_f32x16;
 typedef __attribute__((ext_vector_type(4))) uint32_t gg_u32x4;
 #define GGM_TK 64
 #define GGM_ROW_BYTES 144
-#define GGM_GROUP 8
 
 __device__ __forceinline__ float gg_silu(float g) {
     if (g >= 0.0f) return g / (1.0f + __expf(-g));
@@ -273,32 +272,31 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(
     const int total = tiles_m * tiles_n;
     const int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
     if (logical >= total) return;
-    const int width = GGM_GROUP * tiles_n;
-    const int group = logical / width;
-    const int first_m = group * GGM_GROUP;
-    const int group_size = tiles_m - first_m < GGM_GROUP ? tiles_m - first_m : GGM_GROUP;
-    const int pid_m = first_m + (logical % width) % group_size;
-    const int pid_n = (logical % width) / group_size;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 
-    // the expert of tile pid_m, and the tile's place among that expert's
-    int expert = -1, tile_in_expert = 0;
+    // Workgroups are numbered expert by expert, within an expert feature tile by feature tile, and within that
+    // over the expert's tiles of places: the two or three tiles that read the same rows of W run side by side,
+    // and an expert's places (a megabyte or so) stay in the L2 of the XCD that works through the expert.
+    int expert = -1, tile_in_expert = 0, pid_n = 0;
     {
         int before = 0;
         for (int e0 = 0; e0 < experts; e0 += 64) {
             const int e = e0 + lane;
             const int mine = e < experts ? (expert_begin[e + 1] - expert_begin[e] + TMR - 1) / TMR : 0;
-            int upto = mine;
+            int upto = mine * tiles_n;
 #pragma unroll
             for (int offset = 1; offset < 64; offset <<= 1) {
                 const int other = __shfl_up(upto, offset, 64);
                 if (lane >= offset) upto += other;
             }
-            const unsigned long long holds = __ballot(pid_m < before + upto);
+            const unsigned long long holds = __ballot(logical < before + upto);
             if (holds) {
                 const int at = __ffsll((long long)holds) - 1;
+                const int tiles_here = __shfl(mine, at, 64);
+                const int rest = logical - (before + __shfl(upto, at, 64) - tiles_here * tiles_n);
                 expert = e0 + at;
-                tile_in_expert = pid_m - (before + __shfl(upto, at, 64) - __shfl(mine, at, 64));
+                tile_in_expert = rest % tiles_here;
+                pid_n = rest / tiles_here;
                 break;
             }
             before += __shfl(upto, 63, 64);

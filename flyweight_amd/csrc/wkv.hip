@@ -14,7 +14,9 @@
 // before comes from the same step (normed again here: a row is read twice, nothing is kept between
 // workgroups) or, for a segment's first row, from the request's slot. out[s][row] = h + (before - h) *
 // mu[s]. The workgroup of a segment's FIRST row also moves the slot on to the h of the segment's LAST
-// row: it alone reads and writes the slot, each thread its own channels, the read first.
+// row: it alone reads and writes the slot, each thread its own channels, the read first. A step of few rows
+// has several workgroups a row (blockIdx.y), each with channels of its own (and the row's sums of squares once
+// more): a single token's mixes are then a few loads deep, not one round of loads after the other.
 template <typename T>
 __global__ __launch_bounds__(256) void token_shift_mix_kernel(
     const float* __restrict__ x, const float* __restrict__ norm_weight, float eps, int one_centered,
@@ -37,7 +39,7 @@ __global__ __launch_bounds__(256) void token_shift_mix_kernel(
     const float* other = x + (size_t)(is_first ? last_row : row - 1) * hidden;     // a first row: the row that the slot will hold
     const float inv = inverse_rms(mine);
     const float inv_other = (is_first && last_row == row) ? inv : inverse_rms(other);
-    for (int i = threadIdx.x; i < hidden; i += 256) {
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < hidden; i += 256 * gridDim.y) {
         const float w = norm_weight ? (one_centered ? 1.0f + norm_weight[i] : norm_weight[i]) : 1.0f;
         const float h = mine[i] * inv * w;
         const float h_other = other[i] * inv_other * w;
@@ -59,11 +61,13 @@ extern "C" int fw_token_shift_mix(const float* x, const float* norm_weight, floa
     FW_REQUIRE(rows <= 1 << 20, "token_shift_mix: too many rows (%d)", rows);
     if (rows == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    const int parts = rows <= 128 ? (fw_ceil_div(hidden, 256) < 16 ? fw_ceil_div(hidden, 256) : 16) : 1;
+    const dim3 grid(rows, parts);
     if (out_dtype == FW_F32)
-        token_shift_mix_kernel<float><<<rows, 256, 0, s>>>(x, norm_weight, eps, one_centered, mu, mixes, last, row_seg, seg_row0, seg_slot,
+        token_shift_mix_kernel<float><<<grid, 256, 0, s>>>(x, norm_weight, eps, one_centered, mu, mixes, last, row_seg, seg_row0, seg_slot,
                                                            (float*)out, rows, hidden);
     else if (out_dtype == FW_BF16)
-        token_shift_mix_kernel<bf16_t><<<rows, 256, 0, s>>>(x, norm_weight, eps, one_centered, mu, mixes, last, row_seg, seg_row0, seg_slot,
+        token_shift_mix_kernel<bf16_t><<<grid, 256, 0, s>>>(x, norm_weight, eps, one_centered, mu, mixes, last, row_seg, seg_row0, seg_slot,
                                                             (bf16_t*)out, rows, hidden);
     else
         FW_REQUIRE(false, "token_shift_mix: unknown dtype %d", out_dtype);
@@ -95,7 +99,8 @@ extern "C" int fw_tanh_rows(const float* x, void* out, int out_dtype, long long 
 // sixteen lanes read sixteen neighbouring floats of r, k and the decay from LDS; channels from dim on hold
 // zeros), so that a head is spread over many compute units: the walk along the tokens is one dependent
 // chain per column (a single multiply-add per key channel and token), and only its width can be bought.
-// Tokens come in chunks of WKV_CHUNK (16, fewer for wide heads, whose tokens are larger). A chunk's r, k, a and its block's 16 values travel from global
+// Tokens come in chunks of WKV_CHUNK (16, fewer for wide heads, whose tokens are larger). A chunk's r, k, a
+// and its block's 16 values travel from global
 // memory into registers while the chunk before is walked; on their way into LDS the decay's two
 // exponentials are taken, once per chunk and key channel. A column's sums over key channels (the read-out
 // S^T r and the bonus r . (u k), which every column forms for itself) are each thread's own sum and then
@@ -123,68 +128,68 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
     float* __restrict__ out, const int32_t* __restrict__ seg_row0, const int32_t* __restrict__ seg_slot, int heads, int dim) {
     constexpr int DP = WKV_LANES * RPT;                 // key channels as the lanes hold them
     constexpr int TOKEN = 3 * DP + WKV_COLUMNS;         // a staged token: r, k, decay, the block's values
-    constexpr int PIECES = (WKV_CHUNK * TOKEN + 255) / 256;
+    constexpr int PIECES = (WKV_CHUNK * DP + 255) / 256;    // elements of a chunk's r (and k, and a) per thread, at most
     __shared__ float staged[WKV_CHUNK * TOKEN];
     __shared__ float results[WKV_CHUNK * WKV_COLUMNS];
-    __shared__ float w0s[DP];                           // the decay's offsets of this head
-    static_assert(WKV_CHUNK * WKV_COLUMNS <= 256, "a chunk's read-outs are at most one per thread");
+    static_assert(WKV_CHUNK * WKV_COLUMNS <= 256, "a chunk's read-outs and values are at most one per thread");
     const int seg = blockIdx.x, head = blockIdx.y, block = blockIdx.z;
     const int local = threadIdx.x / WKV_LANES, part = threadIdx.x % WKV_LANES;
     const int column = block * WKV_COLUMNS + local;
     const bool live = column < dim;
     const int first = seg_row0[seg], count = seg_row0[seg + 1] - first;
     const size_t head_at = (size_t)head * dim;
-    // this thread's pieces of every chunk, one float each: token of the chunk, array (0 r, 1 k, 2 a, 3 v) and channel
-    const int per_token = 3 * dim + WKV_COLUMNS;
-    int piece[PIECES];
+    // This thread's elements of every chunk: element e = thread + 256 i of the chunk's [tokens][dim] block of r,
+    // of k and of a alike (token e / dim, channel e % dim), and one of the block's values (token thread / 16,
+    // column thread % 16). A token of -1: no such element.
+    int piece_token[PIECES], piece_channel[PIECES];
+    float piece_w0[PIECES];
 #pragma unroll
     for (int i = 0; i < PIECES; ++i) {
-        const int item = threadIdx.x + 256 * i;
-        const int token = item / per_token, f = item % per_token;
-        int which = f / dim, channel = f % dim;
-        if (which >= 3) {
-            which = 3;
-            channel = f - 3 * dim;
-            if (block * WKV_COLUMNS + channel >= dim) which = 4;     // a column past the head: no such value
-        }
-        piece[i] = token < WKV_CHUNK ? (token << 16) | (which << 12) | channel : -1;
+        const int e = threadIdx.x + 256 * i;
+        const bool there = e < WKV_CHUNK * dim;
+        piece_token[i] = there ? e / dim : -1;
+        piece_channel[i] = there ? e % dim : 0;
+        piece_w0[i] = w0[head_at + piece_channel[i]];
     }
+    const int value_column = block * WKV_COLUMNS + threadIdx.x % WKV_COLUMNS;
+    const int value_token = (threadIdx.x / WKV_COLUMNS < WKV_CHUNK && value_column < dim) ? threadIdx.x / WKV_COLUMNS : -1;
     const int staged_tokens = count < WKV_CHUNK ? count : WKV_CHUNK;        // a decode step stages one token
     for (int i = threadIdx.x; i < staged_tokens * TOKEN; i += 256) staged[i] = 0.0f;
-    for (int i = threadIdx.x; i < DP; i += 256) w0s[i] = i < dim ? w0[head_at + i] : 0.0f;
-    float held[PIECES];
-    // Loads are unconditional (a piece past the chunk's end is read from a valid place again and never used):
-    // behind a branch the compiler would wait for each load at once, and the next chunk would not travel while
-    // this one is walked.
+    float held_r[PIECES], held_k[PIECES], held_a[PIECES], held_v;
+    // Loads are unconditional and their addresses plain arithmetic (an element past the chunk's end, or one that
+    // this thread does not have, is read from a valid place again and never used): behind a branch the compiler
+    // would wait for each load at once, and the next chunk would not travel while this one is walked.
     auto ask = [&](int base) {
         const int last = (count - base < WKV_CHUNK ? count - base : WKV_CHUNK) - 1;
+        const float* r0 = r + (size_t)(first + base) * rkv_stride + head_at;
+        const float* k0 = k + (size_t)(first + base) * rkv_stride + head_at;
+        const float* v0 = v + (size_t)(first + base) * rkv_stride + head_at;
+        const float* a0 = a + (size_t)(first + base) * a_stride + head_at;
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            const int code = piece[i] < 0 ? 0 : piece[i];
-            int token = code >> 16;
+            int token = piece_token[i] < 0 ? 0 : piece_token[i];
             token = token < last ? token : last;
-            const int which = (code >> 12) & 7, channel = code & 0xfff;
-            const size_t row = (size_t)(first + base + token);
-            const float* from = which == 0 ? r + row * rkv_stride + head_at + channel
-                              : which == 1 ? k + row * rkv_stride + head_at + channel
-                              : which == 2 ? a + row * a_stride + head_at + channel
-                              : which == 3 ? v + row * rkv_stride + head_at + block * WKV_COLUMNS + channel
-                                           : r + row * rkv_stride + head_at;
-            held[i] = *from;
+            held_r[i] = r0[token * rkv_stride + piece_channel[i]];
+            held_k[i] = k0[token * rkv_stride + piece_channel[i]];
+            held_a[i] = a0[token * a_stride + piece_channel[i]];
         }
+        int token = value_token < 0 ? 0 : value_token;
+        token = token < last ? token : last;
+        held_v = v0[token * rkv_stride + (value_token < 0 ? 0 : value_column)];
     };
     auto put = [&](int base) {
         const int tokens = count - base < WKV_CHUNK ? count - base : WKV_CHUNK;
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
-            const int code = piece[i];
-            if (code < 0 || (code >> 16) >= tokens) continue;
-            const int token = code >> 16, which = (code >> 12) & 7, channel = code & 0xfff;
-            if (which == 4) continue;
-            float value = held[i];
-            if (which == 2) value = expf(-expf(value + w0s[channel]));
-            staged[token * TOKEN + (which < 3 ? which * DP + channel : 3 * DP + channel)] = value;
+            const float decay = expf(-expf(held_a[i] + piece_w0[i]));
+            if (piece_token[i] >= 0 && piece_token[i] < tokens) {
+                float* to = staged + piece_token[i] * TOKEN + piece_channel[i];
+                to[0] = held_r[i];
+                to[DP] = held_k[i];
+                to[2 * DP] = decay;
+            }
         }
+        if (value_token >= 0 && value_token < tokens) staged[value_token * TOKEN + 3 * DP + threadIdx.x % WKV_COLUMNS] = held_v;
     };
     ask(0);
     float* mine = state + ((size_t)seg_slot[seg] * heads + head) * dim * dim + (live ? column : 0);
@@ -195,7 +200,7 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
         S[t] = (live && key < dim) ? mine[(size_t)key * dim] : 0.0f;
         bonus[t] = key < dim ? u[head_at + key] : 0.0f;
     }
-    __syncthreads();        // the zeros and the offsets are in place
+    __syncthreads();        // the zeros are in place
     put(0);
     __syncthreads();
     for (int base = 0; base < count; base += WKV_CHUNK) {
