@@ -72,54 +72,70 @@ extern "C" int fw_moe_route(const float* logits, const float* bias, int32_t* cho
 }
 
 // ---- sorting the pairs by expert ------------------------------------------------------------------------
-// One workgroup. Pass 1 counts the pairs of every expert (LDS counters), a scan gives where each expert
-// begins, pass 2 hands out places: a thread takes a contiguous run of pairs, in order, and the runs of one
-// expert follow each other in the order of the threads, so that an expert's places hold its pairs in the
-// order (row, choice). expert_begin [experts + 1]; place_row [pairs]; pair_place [pairs].
+// One workgroup of 16 waves; the pairs are cut into 16 runs, one a wave, in order. Pass 1: every wave counts
+// its run's pairs per expert (LDS counters [wave][expert]). A thread per expert then turns the counts into
+// where the expert begins (a scan over the experts by one thread) and where each wave's pairs of it begin.
+// Pass 2: every wave walks its run 64 pairs at a time; the lanes that chose the same expert number themselves
+// by a prefix count (ballot), one expert after the other, behind the wave's running place for that expert.
+// So an expert's places hold its pairs in the order (row, choice), whatever the timing.
+// expert_begin [experts + 1]; place_row [pairs]; pair_place [pairs].
 #define MOE_ARRANGE_THREADS 1024
-#define MOE_ARRANGE_STAGED 10240        // pairs whose experts are kept in LDS (40 KB)
+#define MOE_ARRANGE_WAVES (MOE_ARRANGE_THREADS / 64)
 __global__ __launch_bounds__(MOE_ARRANGE_THREADS) void moe_arrange_kernel(const int32_t* __restrict__ chosen, int32_t* __restrict__ expert_begin,
                                                                           int32_t* __restrict__ place_row, int32_t* __restrict__ pair_place,
-                                                                          int pairs, int experts, int top, int staged) {
-    extern __shared__ int32_t counts[];         // [experts + 1] begins, then the experts of the first `staged` pairs
-    const int tid = threadIdx.x;
-    for (int e = tid; e <= experts; e += MOE_ARRANGE_THREADS) counts[e] = 0;
+                                                                          int pairs, int experts, int top) {
+    extern __shared__ int32_t counts[];         // [waves][experts] counts, then running places; behind them [experts + 1] begins
+    int32_t* begins = counts + MOE_ARRANGE_WAVES * experts;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int run = ((pairs + MOE_ARRANGE_WAVES - 1) / MOE_ARRANGE_WAVES + 63) / 64 * 64;    // pairs of a wave, whole rounds of 64
+    const int run0 = wave * run, run_end = run0 + run < pairs ? run0 + run : pairs;
+    for (int i = tid; i < MOE_ARRANGE_WAVES * experts; i += MOE_ARRANGE_THREADS) counts[i] = 0;
     __syncthreads();
-    for (int i = tid; i < pairs; i += MOE_ARRANGE_THREADS) atomicAdd(&counts[chosen[i]], 1);
+    for (int i = run0 + lane; i < run_end; i += 64) atomicAdd(&counts[wave * experts + chosen[i]], 1);
+    __syncthreads();
+    for (int e = tid; e < experts; e += MOE_ARRANGE_THREADS) {
+        int total = 0;
+        for (int w = 0; w < MOE_ARRANGE_WAVES; ++w) total += counts[w * experts + e];
+        begins[e] = total;
+    }
     __syncthreads();
     if (tid == 0) {
         int running = 0;
         for (int e = 0; e < experts; ++e) {
-            const int n = counts[e];
-            counts[e] = running;
+            const int n = begins[e];
+            begins[e] = running;
             running += n;
         }
-        counts[experts] = running;
+        begins[experts] = running;
     }
     __syncthreads();
-    for (int e = tid; e <= experts; e += MOE_ARRANGE_THREADS) expert_begin[e] = counts[e];
-    // Places in order: a wave per expert at a time walks all pairs in runs of 64 and numbers those of its
-    // expert by a prefix count over the lanes (ballot), so the order is that of the pairs. The walk is one
-    // dependent read after the other: the pairs' experts are first copied behind the counters in LDS where
-    // they fit (staged > 0), and read from there.
-    int32_t* mine = counts + experts + 1;
-    for (int i = tid; i < staged; i += MOE_ARRANGE_THREADS) mine[i] = chosen[i];
+    for (int e = tid; e <= experts; e += MOE_ARRANGE_THREADS) expert_begin[e] = begins[e];
+    for (int e = tid; e < experts; e += MOE_ARRANGE_THREADS) {
+        int running = begins[e];
+        for (int w = 0; w < MOE_ARRANGE_WAVES; ++w) {
+            const int n = counts[w * experts + e];
+            counts[w * experts + e] = running;
+            running += n;
+        }
+    }
     __syncthreads();
-    const int lane = tid & 63, wave = tid >> 6, waves = MOE_ARRANGE_THREADS / 64;
-    for (int e = wave; e < experts; e += waves) {
-        int next = counts[e];
-        const int end = counts[e + 1];
-        if (next == end) continue;
-        for (int i0 = 0; i0 < pairs && next < end; i0 += 64) {
-            const int i = i0 + lane;
-            const bool is_mine = i < pairs && (i < staged ? mine[i] : chosen[i]) == e;
-            const unsigned long long votes = __ballot(is_mine);
-            if (is_mine) {
-                const int place = next + __popcll(votes & ((1ull << lane) - 1ull));
+    int32_t* next = counts + wave * experts;    // this wave's running place for every expert; only this wave touches it
+    for (int i0 = run0; i0 < run_end; i0 += 64) {
+        const int i = i0 + lane;
+        const int e = i < run_end ? chosen[i] : -1;
+        unsigned long long left = __ballot(e >= 0);
+        while (left) {
+            const int leader = __ffsll((long long)left) - 1;
+            const int expert = __shfl(e, leader, 64);
+            const unsigned long long votes = __ballot(e == expert);
+            const int first = next[expert];
+            if (e == expert) {
+                const int place = first + __popcll(votes & ((1ull << lane) - 1ull));
                 place_row[place] = i / top;
                 pair_place[i] = place;
             }
-            next += __popcll(votes);
+            if (lane == leader) next[expert] = first + __popcll(votes);
+            left &= ~votes;
         }
     }
 }
@@ -128,10 +144,15 @@ extern "C" int fw_moe_arrange(const int32_t* chosen, int32_t* expert_begin, int3
                               int top, void* stream) {
     FW_REQUIRE(rows >= 0 && experts >= 1 && experts <= MOE_MAX_EXPERTS && top >= 1, "moe_arrange: bad sizes rows=%d experts=%d top=%d", rows, experts, top);
     FW_REQUIRE((long long)rows * top < (1ll << 30), "moe_arrange: too many pairs");
-    const int pairs = rows * top;
-    const int staged = pairs <= MOE_ARRANGE_STAGED ? pairs : MOE_ARRANGE_STAGED;
-    moe_arrange_kernel<<<1, MOE_ARRANGE_THREADS, (experts + 1 + staged) * sizeof(int32_t), (hipStream_t)stream>>>(
-        chosen, expert_begin, place_row, pair_place, pairs, experts, top, staged);
+    const int lds_bytes = (MOE_ARRANGE_WAVES * experts + experts + 1) * (int)sizeof(int32_t);
+    static int configured = 0;
+    if (lds_bytes > 48 * 1024 && lds_bytes > configured) {
+        hipError_t status = hipFuncSetAttribute((const void*)moe_arrange_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        FW_REQUIRE(status == hipSuccess, "moe_arrange: cannot reserve %d bytes of LDS: %s", lds_bytes, hipGetErrorString(status));
+        configured = lds_bytes;
+    }
+    moe_arrange_kernel<<<1, MOE_ARRANGE_THREADS, lds_bytes, (hipStream_t)stream>>>(chosen, expert_begin, place_row, pair_place, rows * top,
+                                                                                  experts, top);
     FW_LAUNCH_CHECK("moe_arrange");
     return 0;
 }
