@@ -291,7 +291,7 @@ def decode_run(torch, model, config, batch: int, steps: int, warmup: int, seed: 
     elapsed = time.perf_counter() - began
     mean_context = before + 1 + (steps - 1) / 2.0      # keys a row sees, averaged over requests and steps
     cache = runtime.stepper.cache
-    step_bytes = accounting.step_weight_bytes(model.model) + batch * (
+    step_bytes = accounting.step_weight_bytes(model.model, rows=batch) + batch * (
         mean_context * accounting.cache_bytes_per_token(cache) + accounting.state_bytes_per_request(cache))
     runtime.close()
     return elapsed, mean_context, step_bytes

@@ -48,18 +48,38 @@ def _bytes(tensors) -> int:
     return sum(t.numel() * t.element_size() for t in tensors)
 
 
-def step_weight_bytes(model) -> int:
-    """Bytes of every weight a decode step reads once: the layers, the final norm and the head
-    (a tied embedding table is read as the head; an untied one only by the row, which is not
-    counted). ``model``: a bound CausalLM."""
-    return _bytes(_tensors([model.layers, model.final_norm, model.head]))
+def _chosen_parts(model) -> List:
+    """The parts that read only the weights a step's tokens choose (a mixture of experts): they keep those
+    weights out of the walk (``gathered_tensors``) and say themselves what a step reads and a token computes."""
+    found = []
+
+    def visit(part) -> None:
+        if hasattr(part, "chosen_weight_bytes"):
+            found.append(part)
+        for below in (part.sub_parts() if hasattr(part, "sub_parts") else ()):
+            visit(below)
+
+    for block in model.layers:
+        for part in block.parts():
+            visit(part)
+    return found
+
+
+def step_weight_bytes(model, rows: int = 1) -> int:
+    """Bytes of every weight a decode step of ``rows`` tokens reads once: the layers, the final norm and
+    the head (a tied embedding table is read as the head; an untied one only by the row, which is not
+    counted); of weights that tokens choose among, those that ``rows`` tokens are expected to choose.
+    ``model``: a bound CausalLM."""
+    return _bytes(_tensors([model.layers, model.final_norm, model.head])) + sum(
+        int(part.chosen_weight_bytes(rows)) for part in _chosen_parts(model))
 
 
 def product_flops_per_token(model) -> int:
     """Flops of the layers' matrix products for one token (the head is not among them: it runs
     for wanted rows only)."""
     linears = {id(item): item for item in _walk(model.layers, set()) if isinstance(item, Linear)}
-    return 2 * sum(linear.weight.numel() for linear in linears.values())
+    return 2 * sum(linear.weight.numel() for linear in linears.values()) + sum(
+        int(part.chosen_flops_per_token()) for part in _chosen_parts(model))
 
 
 def head_flops_per_row(model) -> int:

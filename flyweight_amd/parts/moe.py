@@ -79,6 +79,19 @@ class MoeSwiGLU(FeedForward):
         if self.shared is not None:
             self.shared.bind(tensors, dtype, device)
 
+    # ----- what a step reads and computes (the experts' weights are read only where tokens chose them) --------
+    def gathered_tensors(self):
+        return (self.gate_up, self.down)
+
+    def chosen_weight_bytes(self, rows: int) -> float:
+        """Bytes of the experts that ``rows`` tokens are expected to choose, each ``top`` different ones and
+        every expert as likely as any other: experts * (1 - (1 - top / experts) ** rows) of them."""
+        per_expert = (self.gate_up[0].numel() + self.down[0].numel()) * self.gate_up.element_size()
+        return self.experts * (1.0 - (1.0 - self.top / self.experts) ** max(int(rows), 0)) * per_expert
+
+    def chosen_flops_per_token(self) -> int:
+        return 2 * self.top * 3 * self.hidden * self.intermediate
+
     def route(self, h: torch.Tensor):
         """(chosen [rows, top], weight [rows, top]) of the rows ``h``."""
         logits = self.router.forward(h, out_dtype=torch.float32)
