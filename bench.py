@@ -119,10 +119,10 @@ def vavelorn_configs(size: dict):
 # sizes, beside the engine's closest existing model: a Koketar of the same width, depth and vocabulary whose dense
 # feed-forward is as wide as the units a Dalerax token runs through (the chosen experts and the shared one).
 DALERAX_SIZES = {
-    "w1024": dict(width=1024, layers=4, vocab=32768, ff=4096, heads=8, kv_heads=2, dim=128, vdim=128, window=512, keep_first=4,
+    "w1024": dict(width=1024, layers=4, vocab=32768, ff=4096, heads=8, kv_heads=2, dim=128, vdim=128, window=512, keep_first=16,
                   rot_dims=64, r_heads=8, r_kv_heads=4, r_dim=64, r_vdim=128, conv=4, rank=32, w_heads=16, w_dim=64,
                   experts=16, top=4, expert_ff=768, shared_ff=1024),
-    "w2048": dict(width=2048, layers=4, vocab=32768, ff=8192, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, keep_first=4,
+    "w2048": dict(width=2048, layers=4, vocab=32768, ff=8192, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, keep_first=16,
                   rot_dims=64, r_heads=16, r_kv_heads=8, r_dim=128, r_vdim=128, conv=4, rank=64, w_heads=32, w_dim=64,
                   experts=32, top=4, expert_ff=1536, shared_ff=2048),
 }
@@ -137,7 +137,7 @@ def dalerax_configs(size: dict):
     attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"],
                  "scale": size["dim"] ** -0.5, "mask": {"size": size["window"], "keep_first": size["keep_first"]},
                  "rot": {"dims": size["rot_dims"], "base": 1000000.0,
-                         "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 2048}}}
+                         "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 2048}}}
     recurrence = {"heads": size["w_heads"], "dim": size["w_dim"], "decay_rank": size["rank"]}
     kinds = [
         {"type": "wkv", "mixer": recurrence, "mlp": dense},

@@ -350,3 +350,31 @@ def test_attention_with_a_sink_against_the_plain_heads(ops, dtype, H, G, d, dv, 
         limit = 2e-5 if dtype == torch.float32 else 2e-2
         for found in every_kernel(ops, q, H, G, d, dv, k_pages, v_pages, ints([pages]), position, scale, window, keep_first, dev(sink), dtype):
             assert np.abs(found - expected[position]).max() <= limit * max(1.0, np.abs(expected[position]).max()), f"position {position}"
+
+
+@pytest.mark.parametrize("H,G,d,dv,window,keep_first", [(4, 2, 32, 48, 40, 3), (6, 3, 16, 16, 33, 70), (2, 1, 64, 128, 1, 2), (8, 2, 64, 64, 64, 1)])
+def test_prompt_attention_with_kept_keys_and_a_sink_over_whole_tiles(ops, H, G, d, dv, window, keep_first):
+    """A prompt of 200 rows in one call of the matrix-core prompt kernel (tiles of 64 rows: a window's edge and the
+    kept keys' edge lie inside tiles and across pages), and its rows from 130 on as a portion behind cached keys;
+    scores with a spread of several units, so that a key wrongly seen or missed moves the output."""
+    T = 200
+    rng = np.random.default_rng(H * d + window)
+    pages = [3, 1, 0, 2]
+    dtype = torch.bfloat16
+    q_all = host(dev(rng.normal(size=(T, H, d)), dtype)).reshape(T, H, d)
+    keys = host(dev(rng.normal(size=(T, G, d)), dtype)).reshape(T, G, d)
+    values = host(dev(rng.normal(size=(T, G, dv)), dtype)).reshape(T, G, dv)
+    sink = rng.normal(size=H) * 2
+    scale = 3.0 * d ** -0.5
+    expected = plain.sink_heads(q_all, keys, values, scale, window, keep_first, sink).reshape(T, H * dv)
+    k_pages, v_pages = paged(keys, values, dtype, pages)
+    for first in (0, 130):
+        seg_row0 = [0, T - first]
+        tile_seg, tile_row0 = ops.query_tiles(seg_row0)
+        q = dev(q_all[first:].reshape(T - first, H * d), dtype)
+        found = ops.attention_prefill(q, H, G, d, k_pages, v_pages, ints([pages]), ints(tile_seg), ints(tile_row0), ints(seg_row0),
+                                      ints(np.arange(first, T)), scale, window, v_dim=dv, keep_first=keep_first, sinks=dev(sink))
+        assert np.abs(host(found) - expected[first:]).max() <= 2e-2 * max(1.0, np.abs(expected).max()), f"rows from {first}"
+        generic = ops.attention_generic(q, H, G, d, k_pages, v_pages, ints([pages]), ints(np.zeros(T - first)), ints(np.arange(first, T)),
+                                        scale, window, v_dim=dv, keep_first=keep_first, sinks=dev(sink))
+        assert np.abs(host(generic) - expected[first:]).max() <= 2e-2 * max(1.0, np.abs(expected).max()), f"plain kernel, rows from {first}"
