@@ -207,6 +207,8 @@ def plain_grouped(a, rows_of_places, w, begin, gated):
     (300, 4, 2, 96, 200),       # hundreds of places an expert: tiles of 128, the last one not full
     (70, 9, 4, 50, 12),         # K no multiple of 8: the plain form in either dtype
     (129, 2, 1, 264, 136),      # one place more than a tile
+    (200, 130, 3, 64, 40),      # more experts than a wave has lanes
+    (2100, 70, 2, 32, 72),      # tiles of 128 places over more than 64 experts, K of half a slab
 ])
 def test_grouped_gemm(ops, dtype, rows, experts, top, K, N):
     rng = np.random.default_rng(rows + N)
