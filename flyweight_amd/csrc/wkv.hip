@@ -95,11 +95,10 @@ extern "C" int fw_tanh_rows(const float* x, void* out, int out_dtype, long long 
 
 // ---- the recurrence ------------------------------------------------------------------------------
 // Workgroup (segment, head, block of 16 value channels); thread = 16 * column + part: a column of S is
-// shared out over the 16 lanes of a row of the wave, RPT key channels each (part, part + 16, ...: the
-// sixteen lanes read sixteen neighbouring floats of r, k and the decay from LDS; channels from dim on hold
-// zeros), so that a head is spread over many compute units: the walk along the tokens is one dependent
+// shared out over the 16 lanes of a row of the wave, RPT neighbouring key channels each (a lane reads its
+// channels of r, of k and of the decay from LDS in one access each; channels from dim on hold zeros), so that a head is spread over many compute units: the walk along the tokens is one dependent
 // chain per column (a single multiply-add per key channel and token), and only its width can be bought.
-// Tokens come in chunks of WKV_CHUNK (16, fewer for wide heads, whose tokens are larger). A chunk's r, k, a
+// Tokens come in chunks of WKV_CHUNK (32, fewer for wide heads, whose tokens are larger). A chunk's r, k, a
 // and its block's 16 values travel from global
 // memory into registers while the chunk before is walked; on their way into LDS the decay's two
 // exponentials are taken, once per chunk and key channel. A column's sums over key channels (the read-out
@@ -129,9 +128,9 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
     constexpr int DP = WKV_LANES * RPT;                 // key channels as the lanes hold them
     constexpr int TOKEN = 3 * DP + WKV_COLUMNS;         // a staged token: r, k, decay, the block's values
     constexpr int PIECES = (WKV_CHUNK * DP + 255) / 256;    // elements of a chunk's r (and k, and a) per thread, at most
-    __shared__ float staged[WKV_CHUNK * TOKEN];
+    __shared__ __attribute__((aligned(16))) float staged[WKV_CHUNK * TOKEN];
     __shared__ float results[WKV_CHUNK * WKV_COLUMNS];
-    static_assert(WKV_CHUNK * WKV_COLUMNS <= 256, "a chunk's read-outs and values are at most one per thread");
+    constexpr int VALUE_PIECES = (WKV_CHUNK * WKV_COLUMNS + 255) / 256;     // of the block's values of a chunk per thread
     const int seg = blockIdx.x, head = blockIdx.y, block = blockIdx.z;
     const int local = threadIdx.x / WKV_LANES, part = threadIdx.x % WKV_LANES;
     const int column = block * WKV_COLUMNS + local;
@@ -152,10 +151,15 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
         piece_w0[i] = w0[head_at + piece_channel[i]];
     }
     const int value_column = block * WKV_COLUMNS + threadIdx.x % WKV_COLUMNS;
-    const int value_token = (threadIdx.x / WKV_COLUMNS < WKV_CHUNK && value_column < dim) ? threadIdx.x / WKV_COLUMNS : -1;
+    int value_token[VALUE_PIECES];
+#pragma unroll
+    for (int j = 0; j < VALUE_PIECES; ++j) {
+        const int token = (threadIdx.x + 256 * j) / WKV_COLUMNS;
+        value_token[j] = (token < WKV_CHUNK && value_column < dim) ? token : -1;
+    }
     const int staged_tokens = count < WKV_CHUNK ? count : WKV_CHUNK;        // a decode step stages one token
     for (int i = threadIdx.x; i < staged_tokens * TOKEN; i += 256) staged[i] = 0.0f;
-    float held_r[PIECES], held_k[PIECES], held_a[PIECES], held_v;
+    float held_r[PIECES], held_k[PIECES], held_a[PIECES], held_v[VALUE_PIECES];
     // Loads are unconditional and their addresses plain arithmetic (an element past the chunk's end, or one that
     // this thread does not have, is read from a valid place again and never used): behind a branch the compiler
     // would wait for each load at once, and the next chunk would not travel while this one is walked.
@@ -173,9 +177,12 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
             held_k[i] = k0[token * rkv_stride + piece_channel[i]];
             held_a[i] = a0[token * a_stride + piece_channel[i]];
         }
-        int token = value_token < 0 ? 0 : value_token;
-        token = token < last ? token : last;
-        held_v = v0[token * rkv_stride + (value_token < 0 ? 0 : value_column)];
+#pragma unroll
+        for (int j = 0; j < VALUE_PIECES; ++j) {
+            int token = value_token[j] < 0 ? 0 : value_token[j];
+            token = token < last ? token : last;
+            held_v[j] = v0[token * rkv_stride + (value_token[j] < 0 ? 0 : value_column)];
+        }
     };
     auto put = [&](int base) {
         const int tokens = count - base < WKV_CHUNK ? count - base : WKV_CHUNK;
@@ -189,14 +196,16 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
                 to[2 * DP] = decay;
             }
         }
-        if (value_token >= 0 && value_token < tokens) staged[value_token * TOKEN + 3 * DP + threadIdx.x % WKV_COLUMNS] = held_v;
+#pragma unroll
+        for (int j = 0; j < VALUE_PIECES; ++j)
+            if (value_token[j] >= 0 && value_token[j] < tokens) staged[value_token[j] * TOKEN + 3 * DP + threadIdx.x % WKV_COLUMNS] = held_v[j];
     };
     ask(0);
     float* mine = state + ((size_t)seg_slot[seg] * heads + head) * dim * dim + (live ? column : 0);
     float S[RPT], bonus[RPT];
 #pragma unroll
     for (int t = 0; t < RPT; ++t) {
-        const int key = t * WKV_LANES + part;
+        const int key = part * RPT + t;
         S[t] = (live && key < dim) ? mine[(size_t)key * dim] : 0.0f;
         bonus[t] = key < dim ? u[head_at + key] : 0.0f;
     }
@@ -213,9 +222,9 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
             const float* t0 = staged + token * TOKEN;
 #pragma unroll
             for (int t = 0; t < RPT; ++t) {
-                r_next[t] = t0[t * WKV_LANES + part];
-                k_next[t] = t0[DP + t * WKV_LANES + part];
-                w_next[t] = t0[2 * DP + t * WKV_LANES + part];
+                r_next[t] = t0[part * RPT + t];
+                k_next[t] = t0[DP + part * RPT + t];
+                w_next[t] = t0[2 * DP + part * RPT + t];
             }
             v_next = t0[3 * DP + local];
         };
@@ -237,10 +246,10 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
         // (barriers that order LDS traffic only: the next chunk's loads stay in flight across them)
         fw_lds_barrier();
         // the chunk's read-outs leave together: a token's 16 columns side by side
-        {
-            const int token = threadIdx.x / WKV_COLUMNS, c = threadIdx.x % WKV_COLUMNS;
-            if (token < tokens && block * WKV_COLUMNS + c < dim)
-                out[((size_t)first + base + token) * heads * dim + head_at + block * WKV_COLUMNS + c] = results[threadIdx.x];
+        for (int i = threadIdx.x; i < tokens * WKV_COLUMNS; i += 256) {
+            const int token = i / WKV_COLUMNS, c = i % WKV_COLUMNS;
+            if (block * WKV_COLUMNS + c < dim)
+                out[((size_t)first + base + token) * heads * dim + head_at + block * WKV_COLUMNS + c] = results[i];
         }
         if (more) put(base + WKV_CHUNK);
         fw_lds_barrier();
@@ -248,7 +257,7 @@ __global__ __launch_bounds__(256) void wkv_recurrence_kernel(
     if (live) {
 #pragma unroll
         for (int t = 0; t < RPT; ++t) {
-            const int key = t * WKV_LANES + part;
+            const int key = part * RPT + t;
             if (key < dim) mine[(size_t)key * dim] = S[t];
         }
     }
@@ -265,9 +274,12 @@ extern "C" int fw_wkv_recurrence(const float* r, const float* k, const float* v,
     hipStream_t s = (hipStream_t)stream;
 #define FW_WKV_LAUNCH(RPT, CHUNK) \
     wkv_recurrence_kernel<RPT, CHUNK><<<grid, 256, 0, s>>>(r, k, v, rkv_stride, a, a_stride, w0, u, state, out, seg_row0, seg_slot, heads, dim)
-    if (dim <= 16) FW_WKV_LAUNCH(1, 16);
-    else if (dim <= 32) FW_WKV_LAUNCH(2, 16);
-    else if (dim <= 64) FW_WKV_LAUNCH(4, 16);
+    // (the chunk's length changes what is staged together, not one sum: steps of single tokens take short chunks,
+    // whose bookkeeping at the start is a few loads)
+    const bool few = rows <= 4 * segments;
+    if (dim <= 16) { if (few) FW_WKV_LAUNCH(1, 4); else FW_WKV_LAUNCH(1, 32); }
+    else if (dim <= 32) { if (few) FW_WKV_LAUNCH(2, 4); else FW_WKV_LAUNCH(2, 32); }
+    else if (dim <= 64) { if (few) FW_WKV_LAUNCH(4, 4); else FW_WKV_LAUNCH(4, 32); }
     else if (dim <= 128) FW_WKV_LAUNCH(8, 8);
     else FW_WKV_LAUNCH(16, 4);
 #undef FW_WKV_LAUNCH

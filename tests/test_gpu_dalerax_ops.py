@@ -87,13 +87,14 @@ def plain_recurrence(r, k, v, decay, u, S, heads, dim):
 
 @pytest.mark.parametrize("heads,dim", [(3, 4), (2, 24), (4, 64), (1, 100), (2, 128), (1, 256)])
 def test_wkv_recurrence(ops, heads, dim):
-    """Segments of 1, 15, 16, 17 and 40 tokens (a chunk's edges) on slots in no order, from states that are not
-    zero; then every request goes on by one token (the state of the first call carried)."""
+    """Segments of 1, 4, 5, 8, 9, 16, 17, 31, 32, 33 and 70 tokens (the edges of chunks of every length the kernel
+    takes) on slots in no order, from states that are not zero; then every request goes on by one token (the state of
+    the first call carried)."""
     rng = np.random.default_rng(dim)
-    lengths, slots = [1, 15, 16, 17, 40], [4, 0, 5, 2, 1]
+    lengths, slots = [1, 4, 5, 8, 9, 16, 17, 31, 32, 33, 70], [4, 0, 5, 2, 1, 11, 7, 12, 6, 9, 10]
     width, rows = heads * dim, sum(lengths)
     seg_row0, _ = segments_of(lengths)
-    state = rng.normal(size=(6, heads, dim, dim)).astype(np.float32) * 0.3
+    state = rng.normal(size=(13, heads, dim, dim)).astype(np.float32) * 0.3
     w0 = rng.normal(size=width).astype(np.float32) - 1.0
     u = rng.normal(size=width).astype(np.float32)
     device_state = dev(state)
