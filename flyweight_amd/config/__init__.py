@@ -4,6 +4,7 @@ from .lfm2 import Lfm2Config
 from .koketar import KoketarConfig
 from .vavelorn import VavelornConfig
 from .dalerax import DaleraxConfig
+from .telapel import TelapelConfig
 from .registry import (architecture_name, config_from_dict, load_config,
                        register_architecture, registered_architectures)
 
@@ -12,9 +13,10 @@ register_architecture("lfm2", Lfm2Config)
 register_architecture("Koketar", KoketarConfig)
 register_architecture("Vavelorn", VavelornConfig)
 register_architecture("Dalerax", DaleraxConfig)
+register_architecture("Telapel", TelapelConfig)
 
 __all__ = [
     "ConfigError", "LayerSpec", "ModelSpec", "PartSpec", "ScheduleEntry", "default_schedule",
-    "Lfm2Config", "KoketarConfig", "VavelornConfig", "DaleraxConfig", "architecture_name", "config_from_dict", "load_config",
+    "Lfm2Config", "KoketarConfig", "VavelornConfig", "DaleraxConfig", "TelapelConfig", "architecture_name", "config_from_dict", "load_config",
     "register_architecture", "registered_architectures",
 ]

@@ -22,7 +22,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, int interleaved, int width) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, int interleaved, int width,
+    const float* __restrict__ q_row_scale) {
     __shared__ float normed[ATTN_MAX_HEAD_DIM];
     const int row = blockIdx.x;
     const int vec = blockIdx.y;
@@ -42,6 +43,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
     }
     const bool is_query = vec < num_heads;
     const float* weight = is_query ? q_norm_weight : k_norm_weight;
+    // a factor on the row's finished queries (one that depends on the row's position, say); keys take none
+    const float factor = (is_query && q_row_scale) ? q_row_scale[row] : 1.0f;
     float inv = 1.0f;
     if (weight) {
         float sum = 0.0f;
@@ -72,7 +75,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_kernel(
             // one rounding of other * s, then one fused step: the same in every kernel that rotates
             value = fmaf(value, c, is_first ? -(other * s) : other * s);
         }
-        store_from_float(dest, d, value);
+        store_from_float(dest, d, q_row_scale ? value * factor : value);
     }
 }
 
@@ -89,7 +92,8 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
     const float* __restrict__ k_norm_weight, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, int rotary_dim, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
-    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows, int interleaved, int width) {
+    const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int rows, int interleaved, int width,
+    const float* __restrict__ q_row_scale) {
     const int r0 = blockIdx.x * QK_ROWS;
     const int vec = blockIdx.y;
     const int lane = threadIdx.x;
@@ -158,6 +162,7 @@ __global__ __launch_bounds__(64) void qk_norm_rope_kv_write_rows_kernel(
         }
         const float other = __shfl(value, partner & 63, 64);
         if (lane < rotary_dim) value = fmaf(value, c[i], is_first ? -(other * sn[i]) : other * sn[i]);
+        if (is_query && q_row_scale) value *= q_row_scale[row_of[i]];
         T* dest = is_query ? q_out + ((size_t)row_of[i] * num_heads + vec) * head_dim
                            : k_pages + (((size_t)page[i] * num_kv_heads + (vec - num_heads)) * ATTN_PAGE + slot) * head_dim;
         if (active) store_from_float(dest, lane, value);
@@ -170,7 +175,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
                                         const int32_t* block_table, int table_stride, const int32_t* row_seg,
                                         const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                                         int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved,
-                                        int q_only, void* stream) {
+                                        int q_only, const float* q_row_scale, void* stream) {
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0, "qk_norm_rope: bad sizes rows=%d heads=%d kv_heads=%d", rows, num_heads, num_kv_heads);
     FW_REQUIRE(head_dim > 0 && head_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: head_dim %d outside 1..%d", head_dim, ATTN_MAX_HEAD_DIM);
     FW_REQUIRE(v_dim > 0 && v_dim <= ATTN_MAX_HEAD_DIM, "qk_norm_rope: value size %d outside 1..%d", v_dim, ATTN_MAX_HEAD_DIM);
@@ -192,7 +197,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_ROWS_LAUNCH(TI, T)                                                                                     \
     qk_norm_rope_kv_write_rows_kernel<TI, T><<<by_rows, 64, 0, s>>>(                                                 \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows, interleaved, width)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, rows, interleaved, width, q_row_scale)
         if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_ROWS_LAUNCH(float, float);
         else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(float, bf16_t);
         else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_ROWS_LAUNCH(bf16_t, bf16_t);
@@ -204,7 +209,7 @@ extern "C" int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_o
 #define FW_QK_LAUNCH(TI, T)                                                                                          \
     qk_norm_rope_kv_write_kernel<TI, T><<<grid, 64, 0, s>>>(                                                         \
         (const TI*)qkv, (T*)q_out, q_norm_weight, k_norm_weight, eps, cos_table, sin_table, rotary_dim, (T*)k_pages, \
-        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, interleaved, width)
+        (T*)v_pages, block_table, table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, interleaved, width, q_row_scale)
     if (in_dtype == FW_F32 && dtype == FW_F32) FW_QK_LAUNCH(float, float);
     else if (in_dtype == FW_F32 && dtype == FW_BF16) FW_QK_LAUNCH(float, bf16_t);
     else if (in_dtype == FW_BF16 && dtype == FW_BF16) FW_QK_LAUNCH(bf16_t, bf16_t);
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ row_seg,
     const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
-    int chunk, float softcap, int keep_first, const float* __restrict__ sinks) {
+    int chunk, float softcap, int keep_first, const float* __restrict__ sinks, const float* __restrict__ slopes) {
     __shared__ float qs[ATTN_MAX_HEAD_DIM];
     __shared__ float ps[ATTN_PAGE];
     const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -253,6 +258,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
             for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], load_as_float(key, d), dot);
             score = dot * scale;
             if (softcap > 0.0f) score = softcap * tanhf(score / softcap);
+            if (slopes) score -= slopes[head] * (float)(pos - t);      // a bias by distance, behind the cap
         }
         const float new_max = fmaxf(running_max, wave_max(score));
         const float p = valid ? expf(score - new_max) : 0.0f;
@@ -294,7 +300,7 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
                                     const void* v_pages, const int32_t* block_table, int table_stride,
                                     const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                     int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk,
-                                    float softcap, int keep_first, const float* sinks, int page_size, int num_pages, void* stream) {
+                                    float softcap, int keep_first, const float* sinks, const float* slopes, int page_size, int num_pages, void* stream) {
     FW_REQUIRE(chunk >= 0 && softcap >= 0.0f, "attention: chunk %d and soft cap %g must not be negative", chunk, (double)softcap);
     FW_REQUIRE(keep_first >= 0 && (keep_first == 0 || chunk == 0), "attention: %d first keys are kept beside a window, not beside chunks", keep_first);
     FW_REQUIRE(rows >= 0 && num_heads > 0 && num_kv_heads > 0 && num_heads % num_kv_heads == 0,
@@ -310,11 +316,11 @@ extern "C" int fw_attention_generic(const void* q, void* out, int dtype, const v
     if (dtype == FW_F32)
         attention_generic_kernel<float><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const float*)q, (float*)out, (const float*)k_pages, (const float*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, keep_first, sinks);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, keep_first, sinks, slopes);
     else if (dtype == FW_BF16)
         attention_generic_kernel<bf16_t><<<grid, 64, 0, (hipStream_t)stream>>>(
             (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_stride,
-            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, keep_first, sinks);
+            row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, keep_first, sinks, slopes);
     else
         FW_REQUIRE(false, "attention: unknown dtype %d", dtype);
     FW_LAUNCH_CHECK("attention_generic");

@@ -75,7 +75,7 @@ template <int HD, int NH, bool CLEAN_V, bool K_PADDED, bool EARLY_V = false>
 __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t* __restrict__ k_page,
                                             const uint16_t* __restrict__ v_page, int head_dim, int v_dim, float scale_log2,
                                             int lo, int hi, int last_written, int k_stride, int v_stride,
-                                            float cap = 0.0f, float cap_scale = 0.0f, int kept = 0) {
+                                            float cap = 0.0f, float cap_scale = 0.0f, int kept = 0, const float* dist = nullptr) {
     const int lane = threadIdx.x & 63;
     const int i16 = lane & 15, g = lane >> 4;
     // all key loads of the page are issued before the first product
@@ -132,6 +132,17 @@ __device__ __forceinline__ void attend_page(Columns<HD> (&c)[NH], const uint16_t
                     const float e = __builtin_amdgcn_exp2f(s[h][kt][r] * twice);
                     s[h][kt][r] = cap - 2.0f * cap * __builtin_amdgcn_rcpf(1.0f + e);
                 }
+    }
+    // A bias by distance, behind the cap: dist[h] (this lane's column of head set h; null: none) times the
+    // number of keys between the column's own position (`hi`, page-relative) and the key is taken off, in
+    // the units of the raw scores.
+    if (dist) {
+#pragma unroll
+        for (int h = 0; h < NH; ++h)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) s[h][kt][r] = fmaf(-dist[h], (float)(hi - (kt * 16 + g * 4 + r)), s[h][kt][r]);
     }
     // `kept`: the keys below it (page-relative; <= 0: none) are seen as well, whatever `lo` says
     const bool full = __all((lo <= 0 || kept >= lo) && hi >= PAGE - 1) && last_written >= PAGE - 1;
@@ -282,7 +293,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ tile_seg, const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ seg_row0,
     const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale_log2, int window,
-    int chunk, float cap, float cap_scale, int keep_first, const float* __restrict__ sinks) {
+    int chunk, float cap, float cap_scale, int keep_first, const float* __restrict__ sinks, const float* __restrict__ slopes) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     // a key's row in LDS holds HD channels, those past head_dim zero: every lane loads its operand
     constexpr int k_stride = HD + KV_PAD;
@@ -385,6 +396,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
             }
         }
     };
+    // the heads' slopes of a bias by distance, in the units of the raw scores (which scale_log2 turns into the exponent's)
+    float dist[NH];
+#pragma unroll
+    for (int h = 0; h < NH; ++h)
+        dist[h] = (slopes && first_in_group + h < group) ? slopes[kvh * group + first_in_group + h] * 1.4426950408889634f / scale_log2 : 0.0f;
     auto attend = [&](int step, int buffer) {
         const int base = block_of(step) * PAGE;
         if (rows > 0 && base <= wave_hi) {      // a wave whose rows all lie before this page has nothing to add
@@ -392,7 +408,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu((HD <= 64 &
             // a lane without a row computes along with the bounds of the tile's first row (nothing of
             // it is stored): a page that is whole for the rows is then whole for the wave
             attend_page<HD, NH, false, true>(c, kt, kt + k_elems, head_dim, v_dim, scale_log2, my_first - base, my_pos - base, pos_hi - base,
-                            k_stride, v_stride, cap, cap_scale, keep_first - base);
+                            k_stride, v_stride, cap, cap_scale, keep_first - base, slopes ? dist : nullptr);
         }
     };
 
@@ -463,6 +479,7 @@ struct FusedProjections {
     int write_kv;                   // 0: another execution of the layer has stored this step's keys and values already
     int interleaved;                // 0: channel i turns with channel i + rotary_dim / 2; 1: channel 2i with channel 2i + 1
     int width;                      // floats of a row of qkv: queries alone where the keys and values are another layer's
+    const float* q_row_scale;       // [rows] or null: a factor on the row's finished queries
 };
 
 // One head-vector of head_dim channels by one wave: optional RMS norm, then the half-split rotation
@@ -510,7 +527,8 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     uint16_t* k_pages, uint16_t* v_pages, const int32_t* __restrict__ block_table, int table_stride,
     const int32_t* __restrict__ row_seg, const int32_t* __restrict__ row_pos, int num_heads, int num_kv_heads,
     int head_dim, int v_dim, float scale_log2, int window, int chunk, float cap, float cap_scale, int max_splits,
-    const int32_t* __restrict__ decode_work, const FusedProjections fused, int keep_first, const float* __restrict__ sinks) {
+    const int32_t* __restrict__ decode_work, const FusedProjections fused, int keep_first, const float* __restrict__ sinks,
+    const float* __restrict__ slopes) {
     __shared__ f32x4 shared_o[SPLIT_PAGES][HD / 16][64];
     __shared__ float shared_m[SPLIT_PAGES][16], shared_l[SPLIT_PAGES][16];
     __shared__ int ticket_shared;
@@ -563,12 +581,13 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         const int vectors = columns + (stores ? 2 : 0);
         const int slot = pos % PAGE;
         const int own_page = stores ? block_table[(size_t)segment * table_stride + last_block] : 0;
+        const float q_factor = fused.q_row_scale ? fused.q_row_scale[row] : 1.0f;
         for (int v = wave; v < vectors; v += SPLIT_PAGES) {
             if (v < columns) {
                 uint16_t* dest = fused_q[v];
                 norm_rotate_vector(projections + (size_t)(kvh * group + head_tile * 16 + v) * head_dim, fused.q_norm_weight, fused.eps,
                                    cos_row, sin_row, fused.rotary_dim, head_dim, fused_scratch[wave],
-                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(value); }, fused.interleaved);
+                                   [&](int d, float value) { dest[d] = float_to_bf16_bits(fused.q_row_scale ? value * q_factor : value); }, fused.interleaved);
             } else if (v == columns) {
                 uint16_t* dest = k_pages + (((size_t)own_page * num_kv_heads + kvh) * PAGE + slot) * head_dim;
                 norm_rotate_vector(projections + (size_t)(num_heads + kvh) * head_dim, fused.k_norm_weight, fused.eps, cos_row, sin_row,
@@ -587,6 +606,8 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
     } else {
         load_query<HD>(c, q + ((size_t)row * num_heads + head) * head_dim, head_dim, valid);
     }
+    // this lane's column is a head: its slope of a bias by distance, in the units of the raw scores
+    float dist[1] = {slopes ? slopes[head] * 1.4426950408889634f / scale_log2 : 0.0f};
     for (int round = 0; round < rounds; ++round) {
         const int step = first_step + round * SPLIT_PAGES + wave;
         if (step > last_step) break;
@@ -596,7 +617,7 @@ __global__ __launch_bounds__(64 * SPLIT_PAGES) __attribute__((amdgpu_waves_per_e
         const int base = block * PAGE;
         // a lane without a head computes along (q = 0, nothing of it is stored)
         attend_page<HD, 1, true, false, (HD <= 128)>(columns_of_wave, k_pages + at * head_dim, v_pages + at * v_dim, head_dim, v_dim, scale_log2, first - base, pos - base, pos - base,
-                        head_dim, PAGE, cap, cap_scale, keep_first - base);
+                        head_dim, PAGE, cap, cap_scale, keep_first - base, slopes ? dist : nullptr);
     }
     const float l = fw_quad_sum(c.l);
 #pragma unroll
@@ -835,7 +856,7 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
                                     const int32_t* tile_row0, int tiles, const int32_t* seg_row0,
                                     const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim,
                                     int v_dim, float scale, int window, int chunk, float softcap, int keep_first, const float* sinks,
-                                    int page_size, int num_pages, int heads_together, void* stream) {
+                                    const float* slopes, int page_size, int num_pages, int heads_together, void* stream) {
     FW_REQUIRE(keep_first >= 0 && (keep_first == 0 || chunk == 0), "attention_prefill: %d first keys are kept beside a window, not beside chunks", keep_first);
     if (check_common("attention_prefill", rows, num_heads, num_kv_heads, head_dim, v_dim, page_size, window, num_pages, table_stride, chunk, softcap)) return -1;
     const ScoreRule rule = score_rule(scale, softcap);
@@ -864,7 +885,7 @@ extern "C" int fw_attention_prefill(const void* q, void* out, const void* k_page
         attention_prefill_kernel<HD, NH><<<grid, 256, lds_bytes, (hipStream_t)stream>>>(                            \
             (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, block_table,    \
             table_stride, tile_seg, tile_row0, seg_row0, row_pos, num_heads, num_kv_heads, head_dim, v_dim,        \
-            rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, keep_first, sinks);                          \
+            rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, keep_first, sinks, slopes);                  \
     }
     if (widest <= 32) {
         if (heads_together == 4) LAUNCH(32, 4) else LAUNCH(32, 1)
@@ -905,7 +926,7 @@ static int decode_check(int max_splits, int max_context, int* tickets, int ticke
 static int decode_launch(const void* q, void* out, float* partial, int max_splits, const int32_t* decode_work, int* tickets, void* k_pages, void* v_pages,
                          const int32_t* block_table, int table_stride, const int32_t* row_seg, const int32_t* row_pos, int rows,
                          int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                         const FusedProjections& fused, int keep_first, const float* sinks, void* stream) {
+                         const FusedProjections& fused, int keep_first, const float* sinks, const float* slopes, void* stream) {
     if (rows == 0) return 0;
     const ScoreRule rule = score_rule(scale, softcap);
     const int head_tiles = (num_heads / num_kv_heads + 15) / 16;
@@ -915,11 +936,11 @@ static int decode_launch(const void* q, void* out, float* partial, int max_split
     if (fused.qkv)                                                                                                            \
         attention_decode_split_kernel<HD, true><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                          \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused, keep_first, sinks); \
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused, keep_first, sinks, slopes); \
     else                                                                                                                      \
         attention_decode_split_kernel<HD, false><<<grid, 64 * SPLIT_PAGES, 0, (hipStream_t)stream>>>(                         \
             (const uint16_t*)q, (uint16_t*)out, partial, tickets, (uint16_t*)k_pages, (uint16_t*)v_pages, block_table,        \
-            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused, keep_first, sinks)
+            table_stride, row_seg, row_pos, num_heads, num_kv_heads, head_dim, v_dim, rule.scale_log2, window, chunk, rule.cap, rule.cap_scale, max_splits, decode_work, fused, keep_first, sinks, slopes)
     FW_BY_HEAD_DIM((head_dim > v_dim ? head_dim : v_dim), CALL);
 #undef CALL
     FW_LAUNCH_CHECK("attention_decode");
@@ -939,11 +960,11 @@ extern "C" int fw_attention_decode(const void* q, void* out, float* partial, int
                                    const void* v_pages, const int32_t* block_table, int table_stride,
                                    const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                    int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                                   int keep_first, const float* sinks, int page_size, int num_pages, void* stream) {
+                                   int keep_first, const float* sinks, const float* slopes, int page_size, int num_pages, void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
                      page_size, num_pages, chunk, softcap, keep_first)) return -1;
     return decode_launch(q, out, partial, max_splits, decode_work, tickets, const_cast<void*>(k_pages), const_cast<void*>(v_pages), block_table,
-                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, FusedProjections{}, keep_first, sinks, stream);
+                         table_stride, row_seg, row_pos, rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, FusedProjections{}, keep_first, sinks, slopes, stream);
 }
 
 // fw_attention_decode with the work of fw_qk_norm_rope_kv_write in front of it, in the same kernel:
@@ -957,8 +978,8 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
                                          void* k_pages, void* v_pages, const int32_t* block_table, int table_stride,
                                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                                          int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                                         int interleaved, int q_only, int keep_first, const float* sinks, int page_size, int num_pages,
-                                         void* stream) {
+                                         int interleaved, int q_only, int keep_first, const float* sinks, const float* slopes,
+                                         const float* q_row_scale, int page_size, int num_pages, void* stream) {
     if (decode_check(max_splits, max_context, tickets, tickets_len, table_stride, rows, num_heads, num_kv_heads, head_dim, v_dim, window,
                      page_size, num_pages, chunk, softcap, keep_first)) return -1;
     FW_REQUIRE(!(q_only && write_kv), "attention_decode_fused: rows that hold queries only bring no keys or values to store");
@@ -971,7 +992,8 @@ extern "C" int fw_attention_decode_fused(const float* qkv, const float* q_norm_w
     fused.qkv = qkv; fused.q_norm_weight = q_norm_weight; fused.k_norm_weight = k_norm_weight; fused.eps = eps;
     fused.cos_table = cos_table; fused.sin_table = sin_table; fused.rotary_dim = rotary_dim; fused.write_kv = write_kv;
     fused.interleaved = interleaved;
+    fused.q_row_scale = q_row_scale;
     fused.width = q_only ? num_heads * head_dim : (num_heads + num_kv_heads) * head_dim + num_kv_heads * v_dim;
     return decode_launch(nullptr, out, partial, max_splits, decode_work, tickets, k_pages, v_pages, block_table, table_stride, row_seg, row_pos,
-                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, fused, keep_first, sinks, stream);
+                         rows, num_heads, num_kv_heads, head_dim, v_dim, scale, window, chunk, softcap, fused, keep_first, sinks, slopes, stream);
 }

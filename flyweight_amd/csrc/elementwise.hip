@@ -16,7 +16,7 @@ void fw_set_error(const char* format, ...) {
     va_end(args);
 }
 extern "C" const char* fw_last_error(void) { return fw_error_text; }
-extern "C" int fw_abi_version(void) { return 15; }
+extern "C" int fw_abi_version(void) { return 16; }
 
 // ---- embedding -------------------------------------------------------------------------
 // The reference gathers one row per token and widens it to float32
@@ -213,6 +213,23 @@ extern "C" int fw_rope_table(const int32_t* positions, const double* inv_freq, f
     const long long total = (long long)rows * half;
     rope_table_kernel<<<fw_ceil_div(total, 256), 256, 0, (hipStream_t)stream>>>(positions, inv_freq, cos_out, sin_out, rows, half);
     FW_LAUNCH_CHECK("rope_table");
+    return 0;
+}
+
+// ---- a factor on the queries that grows with the position ----------------------------------
+// out[r] = 1 + coef * ln(floor((position + 1) / every) + 1): 1 for the first `every` - 1 positions, then a step up
+// every `every` positions. Float32 (the count is a whole number; its logarithm is float32).
+__global__ void query_temperature_kernel(const int32_t* __restrict__ positions, float* __restrict__ out, int rows, float coef, int every) {
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= rows) return;
+    out[row] = 1.0f + coef * logf((float)((positions[row] + 1) / every + 1));
+}
+
+extern "C" int fw_query_temperature(const int32_t* positions, float* out, int rows, float coef, int every, void* stream) {
+    FW_REQUIRE(rows >= 0 && every > 0, "query_temperature: bad sizes rows=%d every=%d", rows, every);
+    if (rows == 0) return 0;
+    query_temperature_kernel<<<fw_ceil_div(rows, 256), 256, 0, (hipStream_t)stream>>>(positions, out, rows, coef, every);
+    FW_LAUNCH_CHECK("query_temperature");
     return 0;
 }
 

@@ -114,6 +114,9 @@ int fw_swiglu(const void* gate_up, int in_dtype, void* out, int out_dtype, int r
 int fw_rope_table(const int32_t* positions, const double* inv_freq, float* cos_out, float* sin_out,
                   int rows, int half, void* stream);
 
+// out[r] = 1 + coef * ln(floor((positions[r] + 1) / every) + 1): a factor on a row's queries that grows with its position
+int fw_query_temperature(const int32_t* positions, float* out, int rows, float coef, int every, void* stream);
+
 // Gated short convolution over a mixed batch. bcx [rows][3H] = (B | C | x); taps [H][L]
 // oldest first; conv_bias [H] or null; state [slots][H][L-1] float32, oldest first.
 // Row r belongs to segment row_seg[r]; segment s covers rows seg_row0[s]..seg_row0[s+1]
@@ -133,7 +136,8 @@ int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dty
                              const float* sin_table, int rotary_dim, void* k_pages, void* v_pages,
                              const int32_t* block_table, int table_stride, const int32_t* row_seg,
                              const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
-                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved, int q_only, void* stream);
+                             int head_dim, int v_dim, int page_size, int num_pages, int write_kv, int interleaved, int q_only,
+                             const float* q_row_scale, void* stream);
 
 // Causal attention of every row over the cached keys 0..row_pos[r] of its segment, or the last `window`
 // of them, or with `chunk` > 0 those of its own chunk of that many positions (counted from position 0
@@ -142,11 +146,14 @@ int fw_qk_norm_rope_kv_write(const void* qkv, int in_dtype, void* q_out, int dty
 // stands. sinks (float32 [heads], or null): one more term exp(sinks[head]) in the softmax's denominator, with
 // no key and no value, not scaled. (q_only of fw_qk_norm_rope_kv_write / fw_attention_decode_fused: the rows
 // of qkv hold the queries alone, [heads * head_dim]: the keys and values are another layer's.)
+// slopes (float32 [heads], or null): a bias by distance, slopes[head] * (row's position - key's position) is taken off
+// the score behind the cap. q_row_scale (float32 [rows], or null; fw_qk_norm_rope_kv_write and
+// fw_attention_decode_fused): a factor on the row's normed and rotated queries (one that depends on the position, say).
 int fw_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                          const void* v_pages, const int32_t* block_table, int table_stride,
                          const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads,
                          int num_kv_heads, int head_dim, int v_dim, float scale, int window, int chunk, float softcap,
-                         int keep_first, const float* sinks, int page_size, int num_pages, void* stream);
+                         int keep_first, const float* sinks, const float* slopes, int page_size, int num_pages, void* stream);
 
 // The same attention on the matrix cores, bfloat16 only, head_dim and v_dim (the size of a value and of a
 // head's output: out [rows][nh * v_dim]) multiples of 16 up to 256.
@@ -159,7 +166,7 @@ int fw_attention_prefill(const void* q, void* out, const void* k_pages, const vo
                          const int32_t* block_table, int table_stride, const int32_t* tile_seg,
                          const int32_t* tile_row0, int tiles, const int32_t* seg_row0, const int32_t* row_pos,
                          int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim, float scale, int window,
-                         int chunk, float softcap, int keep_first, const float* sinks, int page_size, int num_pages,
+                         int chunk, float softcap, int keep_first, const float* sinks, const float* slopes, int page_size, int num_pages,
                          int heads_together, void* stream);
 // Decode (one row per request): the keys are split between workgroups in runs of 4 pages and
 // merged in order by the workgroup that finishes last. partial: float32 workspace
@@ -172,7 +179,7 @@ int fw_attention_decode(const void* q, void* out, float* partial, int max_splits
                         const int32_t* decode_work, int* tickets, int tickets_len, const void* k_pages, const void* v_pages, const int32_t* block_table, int table_stride,
                         const int32_t* row_seg, const int32_t* row_pos, int rows, int num_heads, int num_kv_heads,
                         int head_dim, int v_dim, float scale, int window, int chunk, float softcap, int keep_first,
-                        const float* sinks, int page_size, int num_pages, void* stream);
+                        const float* sinks, const float* slopes, int page_size, int num_pages, void* stream);
 
 // The same with the work of fw_qk_norm_rope_kv_write in front of it, in one kernel: qkv float32
 // [rows][(heads + kv_heads) * head_dim + kv_heads * v_dim] are the step's raw projections; every workgroup norms and
@@ -185,7 +192,7 @@ int fw_attention_decode_fused(const float* qkv, const float* q_norm_weight, cons
                               void* v_pages, const int32_t* block_table, int table_stride, const int32_t* row_seg,
                               const int32_t* row_pos, int rows, int num_heads, int num_kv_heads, int head_dim, int v_dim,
                               float scale, int window, int chunk, float softcap, int interleaved, int q_only, int keep_first,
-                              const float* sinks, int page_size, int num_pages, void* stream);
+                              const float* sinks, const float* slopes, const float* q_row_scale, int page_size, int num_pages, void* stream);
 
 // ids[r] = argmax(logits[r]) with ties to the lowest id, also written to also[r] if that is not null;
 // advance[r] += 1 if that is not null; workspace: rows * 64 64-bit words
@@ -278,15 +285,26 @@ int fw_clamped_glu(const void* gate_up, int in_dtype, void* out, int out_dtype, 
 // ---- attention over a cached latent ---------------------------------------------------------------
 // The latent of a step's rows: columns col0 .. col0 + rank - 1 of raw [rows][raw_stride] (float32), RMS-normed
 // (eps under the root) times weight [rank], stored at each row's position in both layouts of a cache
-// with one key/value head of `rank` channels: k_pages [pages][1][P][rank], v_pages [pages][1][rank][P].
+// with one key/value head of `rank` channels: k_pages [pages][1][P][rank + rot], v_pages [pages][1][rank][P].
+// rot > 0: the next rot columns of raw are a key part that all heads share: not normed, neighbouring channels
+// (2i, 2i + 1) of its first `turn` turned by the row's angles (tables [rows][turn / 2]), stored behind the latent in the key layout only.
 int fw_latent_norm_write(const float* raw, int raw_stride, int col0, const float* weight, float eps, void* k_pages,
                          void* v_pages, int dtype, const int32_t* block_table, int table_stride, const int32_t* row_seg,
-                         const int32_t* row_pos, int rows, int rank, int page_size, int num_pages, void* stream);
+                         const int32_t* row_pos, int rows, int rank, int rot, int turn, const float* cos_table, const float* sin_table,
+                         int page_size, int num_pages, void* stream);
 // A map per head: out[r][h N + n] = sum_k in[r][h K + k] * w[h][n][k], with a gate (may be null) times
 // sigmoid(gate[r][h N + n]). in [rows][in_stride], w [heads][N][K], gate float32 [rows][gate_stride],
-// out [rows][heads N].
+// out [rows][heads N]. in_head / out_head / out_stride (0: K, N, heads * out_head): a head's inputs lie in_head apart
+// and its outputs out_head apart in rows out_stride wide, where a head's vector holds more than the map reads or writes.
 int fw_head_linear(const void* in, int in_dtype, int in_stride, const void* w, int w_dtype, const float* gate, int gate_stride,
-                   void* out, int out_dtype, int rows, int heads, int N, int K, void* stream);
+                   void* out, int out_dtype, int rows, int heads, int N, int K, int in_head, int out_head, int out_stride,
+                   void* stream);
+// Channels col0 .. col0 + rot - 1 of every head's vector (heads in_head apart in rows in_stride wide) turned, neighbouring
+// channels (2i, 2i + 1) of the first `turn` by the row's angles (tables [rows][turn / 2]), and stored from channel out_col0 of the head's
+// vector in out (heads out_head apart in rows out_stride wide).
+int fw_rotate_place(const void* in, int in_dtype, int in_stride, int in_head, int col0, const float* cos_table,
+                    const float* sin_table, void* out, int out_dtype, int out_stride, int out_head, int out_col0, int rows,
+                    int heads, int rot, int turn, void* stream);
 
 // ---- a recurrence with a decay per key channel formed by the token ("wkv") --------------------------------
 // Token shift: h = rmsnorm(x) * (w or 1 + w) (norm_weight null: h = x); out[s][r] = h[r] + (h[r - 1] - h[r]) * mu[s],
@@ -306,21 +324,44 @@ int fw_wkv_recurrence(const float* r, const float* k, const float* v, int rkv_st
 
 // ---- a mixture of feed-forward units chosen per token ------------------------------------------------------
 // chosen / weight [rows][top]: the `top` largest of logits[r] + bias (float32 [rows][experts]; ties: the lowest
-// id; bias may be null), largest first, and the softmax over those alone.
+// id; bias may be null), largest first, and the softmax over those alone. groups > 1: the experts form that many equal
+// groups of neighbours, a group's score is its best expert's, and only experts of the `keep` best groups (ties: the
+// lowest group) can be chosen. score_all: the weights are the softmax over ALL experts at the chosen ones, divided by
+// their sum + 1e-20.
 int fw_moe_route(const float* logits, const float* bias, int32_t* chosen, float* weight, int rows, int experts, int top,
-                 void* stream);
+                 int groups, int keep, int score_all, void* stream);
 // The pairs (row, choice) sorted by expert, in the order of the pairs within an expert: expert_begin
 // [experts + 1], place_row [rows * top] (the row of each place), pair_place [rows * top] (the place of each pair).
 int fw_moe_arrange(const int32_t* chosen, int32_t* expert_begin, int32_t* place_row, int32_t* pair_place, int rows, int experts,
                    int top, void* stream);
 // out[place] = a[place_row ? place_row[place] : place] . w[expert of place]^T; w [experts][N][K], or with
-// gated [experts][2 N][K] (gate rows, then up rows) and out = silu(gate) * up. out [places][N].
+// gated [experts][2 N][K] (gate rows, then up rows) and out = silu(gate) * up, or with a glu_limit > 0 the clamped
+// unit g sigmoid(glu_alpha g) (u + glu_shift), g = min(gate, limit), u = clamp(up, -limit, limit). out [places][N].
 int fw_grouped_gemm(const void* a, int a_dtype, const int32_t* place_row, const void* w, int w_dtype,
                     const int32_t* expert_begin, void* out, int out_dtype, int gated, int places, int experts, int N, int K,
-                    void* stream);
+                    float glu_limit, float glu_alpha, float glu_shift, void* stream);
 // x[r] += sum_j weight[r][j] * y[pair_place[r][j]], j in order; float32
 int fw_moe_combine(float* x, const float* y, const float* weight, const int32_t* pair_place, int rows, int top, int hidden,
                    void* stream);
+
+// ---- a short causal convolution per channel, and a gated linear recurrence per channel -----------------------------
+// y[t][c] = sum_j taps[c][j] * x[t - L + 1 + j][c] (+ bias[c]; null: none) over mixed segments, float32. in [rows][in_stride]
+// (the first `channels` columns), taps [channels][L] with the last column the current token's, state [slots][channels][L - 1]
+// oldest first: the inputs before a segment's first row, read and then moved on by the segment's rows. out [rows][out_stride];
+// channels echo_col0 .. + echo_cols - 1 are written once more from column echo_to on (echo_cols 0: none). single_rows: every
+// segment is one row (row r is segment r): outputs and the slots' move in one launch.
+int fw_causal_conv(const float* in, int in_stride, const float* taps, const float* bias, float* state, const int32_t* row_seg,
+                   const int32_t* seg_row0, const int32_t* seg_slot, float* out, int out_stride, int echo_col0, int echo_cols,
+                   int echo_to, int rows, int segments, int channels, int taps_count, int slots, int single_rows, void* stream);
+// Per segment and channel c, row by row: r = sigmoid(gates[r_col] + r_bias[c]), i = sigmoid(gates[i_col] + i_bias[c]),
+// a = exp(-rate * r * softplus(lam[c])), S <- a S + sqrt(1 - a^2) * i * u[c], out[c] = S * gelu_tanh(y[c]). The gates of a
+// block of block_width channels lie side by side, [r of the block | i of the block], block after block (gates rows of
+// gates_stride >= 2 * channels floats). state float32 [slots][channels], read at a segment's start, written at its end.
+// All float32; out [rows][channels] of out_dtype.
+int fw_rglru_scan(const float* u, int u_stride, const float* gates, int gates_stride, const float* y, int y_stride,
+                  const float* r_bias, const float* i_bias, const float* lam, float rate, float* state, const int32_t* seg_row0,
+                  const int32_t* seg_slot, void* out, int out_dtype, int rows, int segments, int channels, int block_width,
+                  int slots, void* stream);
 
 #ifdef __cplusplus
 }

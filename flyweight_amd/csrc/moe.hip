@@ -17,14 +17,67 @@
 // MOE_MAX_EXPERTS / 64 a lane; `top` rounds of a wave-wide best-of, each taking the winner out.
 #define MOE_MAX_EXPERTS 1024
 #define MOE_MAX_TOP 64
+// groups > 1: the experts form that many equal groups of neighbours, a group's score is its best expert's, and only
+// experts of the `keep` best groups (ties: the lowest group) can be chosen. score_all: the weights are the softmax
+// over ALL experts at the chosen ones, divided by their sum + 1e-20 (else the softmax over the chosen alone).
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
-                                                      int32_t* __restrict__ chosen, float* __restrict__ weight, int experts, int top) {
+                                                      int32_t* __restrict__ chosen, float* __restrict__ weight, int experts, int top,
+                                                      int groups, int keep, int score_all) {
     const int row = blockIdx.x, lane = threadIdx.x;
     float z[MOE_MAX_EXPERTS / 64];
 #pragma unroll
     for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i) {
         const int e = lane + 64 * i;
         z[i] = e < experts ? logits[(size_t)row * experts + e] + (bias ? bias[e] : 0.0f) : -INFINITY;
+    }
+    float all_max = 0.0f, all_sum = 1.0f;
+    if (score_all) {    // the softmax's maximum and sum over every expert, before any is shut out
+        float m = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i) m = fmaxf(m, z[i]);
+        all_max = wave_max(m);
+        float sum = 0.0f;
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i)
+            if (lane + 64 * i < experts) sum += expf(z[i] - all_max);
+        all_sum = wave_sum(sum);
+    }
+    if (groups > 1 && keep < groups) {
+        // lane g holds the best logit of group g (the softmax is monotonic: the best score is the best logit's)
+        const int per_group = experts / groups;
+        float group_best = -INFINITY;
+        for (int g = 0; g < groups; ++g) {
+            float m = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i) {
+                const int e = lane + 64 * i;
+                if (e < experts && e / per_group == g) m = fmaxf(m, z[i]);
+            }
+            m = wave_max(m);
+            if (lane == g) group_best = m;
+        }
+        unsigned long long kept = 0ull;
+        for (int round = 0; round < keep; ++round) {
+            // a group already taken is no longer offered
+            const bool offered = lane < groups && !((kept >> lane) & 1ull);
+            float best = offered ? group_best : -INFINITY;
+            int best_id = offered ? lane : 0x7fffffff;
+#pragma unroll
+            for (int offset = 32; offset > 0; offset >>= 1) {
+                const float other = __shfl_xor(best, offset, 64);
+                const int other_id = __shfl_xor(best_id, offset, 64);
+                if (other_id < 0x7fffffff && (best_id == 0x7fffffff || other > best || (other == best && other_id < best_id))) {
+                    best = other;
+                    best_id = other_id;
+                }
+            }
+            kept |= 1ull << best_id;        // every lane holds the same winner
+        }
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i) {
+            const int e = lane + 64 * i;
+            if (e < experts && !((kept >> (e / per_group)) & 1ull)) z[i] = -INFINITY;
+        }
     }
     float first = 0.0f, total = 0.0f, mine = 0.0f;      // lane j keeps the j-th choice's exponential
     for (int round = 0; round < top; ++round) {
@@ -51,22 +104,27 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
         for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i)
             if (lane + 64 * i == best_id) z[i] = -INFINITY;
         if (round == 0) first = best;                   // the largest: the softmax's shift
-        const float e = expf(best - first);
+        const float e = score_all ? expf(best - all_max) / all_sum : expf(best - first);
         total += e;
         if (lane == round) {
             mine = e;
             chosen[(size_t)row * top + round] = best_id;
         }
     }
-    if (lane < top) weight[(size_t)row * top + lane] = mine / total;
+    if (lane < top) weight[(size_t)row * top + lane] = mine / (score_all ? total + 1e-20f : total);
 }
 
 extern "C" int fw_moe_route(const float* logits, const float* bias, int32_t* chosen, float* weight, int rows, int experts, int top,
-                            void* stream) {
+                            int groups, int keep, int score_all, void* stream) {
+    if (groups <= 0) groups = 1;
+    if (keep <= 0) keep = groups;
+    FW_REQUIRE(groups <= 64 && experts % groups == 0 && keep <= groups, "moe_route: %d experts in %d groups (at most 64, equal ones) of which %d are kept",
+               experts, groups, keep);
+    FW_REQUIRE(top <= keep * (experts / groups), "moe_route: %d experts a token cannot come from %d groups of %d", top, keep, experts / groups);
     FW_REQUIRE(rows >= 0 && experts >= 1 && experts <= MOE_MAX_EXPERTS, "moe_route: %d experts (1..%d)", experts, MOE_MAX_EXPERTS);
     FW_REQUIRE(top >= 1 && top <= experts && top <= MOE_MAX_TOP, "moe_route: %d of %d experts a token (at most %d)", top, experts, MOE_MAX_TOP);
     if (rows == 0) return 0;
-    moe_route_kernel<<<rows, 64, 0, (hipStream_t)stream>>>(logits, bias, chosen, weight, experts, top);
+    moe_route_kernel<<<rows, 64, 0, (hipStream_t)stream>>>(logits, bias, chosen, weight, experts, top, groups, keep, score_all);
     FW_LAUNCH_CHECK("moe_route");
     return 0;
 }
@@ -157,6 +215,16 @@ extern "C" int fw_moe_arrange(const int32_t* chosen, int32_t* expert_begin, int3
     return 0;
 }
 
+// The gated unit of a place: silu(gate) * up, or with a positive limit the clamped form
+// g sigmoid(alpha g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit).
+struct GatedUnit {
+    float limit, alpha, shift;
+};
+__device__ __forceinline__ float gg_clamped(float gate, float up, const GatedUnit unit) {
+    const float g = fminf(gate, unit.limit), u = fminf(fmaxf(up, -unit.limit), unit.limit);
+    return g / (1.0f + expf(-unit.alpha * g)) * (u + unit.shift);
+}
+
 // ---- the grouped product, plain form ------------------------------------------------------------------
 // Tiles of GG_ROWS places x GG_COLS features; a tile's places belong to one expert. blockIdx.x numbers
 // the row tiles of all experts one after the other (an expert with n places has ceil(n / GG_ROWS)); the
@@ -169,7 +237,7 @@ extern "C" int fw_moe_arrange(const int32_t* chosen, int32_t* expert_begin, int3
 template <typename TA, typename TW, typename TO, bool GATED>
 __global__ __launch_bounds__(256) void grouped_gemm_kernel(const TA* __restrict__ a, const int32_t* __restrict__ place_row,
                                                           const TW* __restrict__ w, const int32_t* __restrict__ expert_begin,
-                                                          TO* __restrict__ out, int experts, int N, int K) {
+                                                          TO* __restrict__ out, int experts, int N, int K, const GatedUnit unit) {
     __shared__ float as[GG_K][GG_ROWS + 1];
     __shared__ float ws[GATED ? 2 : 1][GG_K][GG_COLS + 1];
     __shared__ int tile_expert, tile_first, tile_end;
@@ -243,7 +311,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(const TA* __restrict_
             float value = acc[0][i][j];
             if (GATED) {
                 const float g = acc[0][i][j];
-                value = g / (1.0f + expf(-g)) * acc[1][i][j];
+                value = unit.limit > 0.0f ? gg_clamped(g, acc[1][i][j], unit) : g / (1.0f + expf(-g)) * acc[1][i][j];
             }
             store_from_float(out, (size_t)(first + r) * N + col, value);
         }
@@ -281,7 +349,8 @@ __device__ __forceinline__ float gg_silu(float g) {
 template <bool GATED, bool BIG, int NJ, typename TO>
 __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(
     const uint16_t* __restrict__ a, const int32_t* __restrict__ place_row, const uint16_t* __restrict__ w,
-    const int32_t* __restrict__ expert_begin, TO* __restrict__ out, int experts, int N, int K, int tiles_m, int tiles_n, int per_xcd) {
+    const int32_t* __restrict__ expert_begin, TO* __restrict__ out, int experts, int N, int K, int tiles_m, int tiles_n, int per_xcd,
+    const GatedUnit unit) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int TMR = BIG ? 128 : 32;                 // places of a tile
     constexpr int WAVES_M = BIG ? 2 : 1, WAVES_N = 4 / WAVES_M;
@@ -458,7 +527,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(
             if (place >= end) continue;
             if (GATED) {
                 const int n = n0 + wn * 32 + col;
-                if (n < N) store_from_float(out, (size_t)place * N + n, gg_silu(acc[i][0][r]) * acc[i][NJ - 1][r]);
+                if (n < N)
+                    store_from_float(out, (size_t)place * N + n, unit.limit > 0.0f ? gg_clamped(acc[i][0][r], acc[i][NJ - 1][r], unit)
+                                                                                    : gg_silu(acc[i][0][r]) * acc[i][NJ - 1][r]);
             } else {
 #pragma unroll
                 for (int j = 0; j < NJ; ++j) {
@@ -471,7 +542,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_mfma_kernel(
 
 template <bool GATED, bool BIG, int NJ, typename TO>
 static int grouped_mfma_launch(const void* a, const int32_t* place_row, const void* w, const int32_t* expert_begin, void* out, int places,
-                               int experts, int N, int K, hipStream_t stream) {
+                               int experts, int N, int K, const GatedUnit unit, hipStream_t stream) {
     constexpr int TMR = BIG ? 128 : 32;
     constexpr int BN = (BIG ? 2 : 4) * NJ * 32;
     const int features = GATED ? BN / 2 : BN;
@@ -488,13 +559,15 @@ static int grouped_mfma_launch(const void* a, const int32_t* place_row, const vo
         configured = true;
     }
     grouped_gemm_mfma_kernel<GATED, BIG, NJ, TO><<<per_xcd * 8, 256, lds_bytes, stream>>>(
-        (const uint16_t*)a, place_row, (const uint16_t*)w, expert_begin, (TO*)out, experts, N, K, (int)tiles_m, (int)tiles_n, per_xcd);
+        (const uint16_t*)a, place_row, (const uint16_t*)w, expert_begin, (TO*)out, experts, N, K, (int)tiles_m, (int)tiles_n, per_xcd, unit);
     return 0;
 }
 
 extern "C" int fw_grouped_gemm(const void* a, int a_dtype, const int32_t* place_row, const void* w, int w_dtype,
                                const int32_t* expert_begin, void* out, int out_dtype, int gated, int places, int experts, int N, int K,
-                               void* stream) {
+                               float glu_limit, float glu_alpha, float glu_shift, void* stream) {
+    const GatedUnit unit = {glu_limit, glu_alpha, glu_shift};
+    FW_REQUIRE(glu_limit <= 0.0f || gated, "grouped_gemm: a clamped unit goes with gate and up rows");
     FW_REQUIRE(places >= 0 && experts >= 1 && N > 0 && K > 0, "grouped_gemm: bad sizes places=%d experts=%d N=%d K=%d", places, experts, N, K);
     if (places == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
@@ -503,10 +576,10 @@ extern "C" int fw_grouped_gemm(const void* a, int a_dtype, const int32_t* place_
         (out_dtype == FW_F32 || (out_dtype == FW_BF16 && gated))) {
         const bool big = (long long)places >= 48ll * experts;
         int status;
-        if (gated) status = big ? grouped_mfma_launch<true, true, 2, bf16_t>(a, place_row, w, expert_begin, out, places, experts, N, K, s)
-                                : grouped_mfma_launch<true, false, 2, bf16_t>(a, place_row, w, expert_begin, out, places, experts, N, K, s);
-        else status = big ? grouped_mfma_launch<false, true, 2, float>(a, place_row, w, expert_begin, out, places, experts, N, K, s)
-                          : grouped_mfma_launch<false, false, 1, float>(a, place_row, w, expert_begin, out, places, experts, N, K, s);
+        if (gated) status = big ? grouped_mfma_launch<true, true, 2, bf16_t>(a, place_row, w, expert_begin, out, places, experts, N, K, unit, s)
+                                : grouped_mfma_launch<true, false, 2, bf16_t>(a, place_row, w, expert_begin, out, places, experts, N, K, unit, s);
+        else status = big ? grouped_mfma_launch<false, true, 2, float>(a, place_row, w, expert_begin, out, places, experts, N, K, unit, s)
+                          : grouped_mfma_launch<false, false, 1, float>(a, place_row, w, expert_begin, out, places, experts, N, K, unit, s);
         if (status != 0) return status;
         FW_LAUNCH_CHECK("grouped_gemm");
         return 0;
@@ -517,9 +590,9 @@ extern "C" int fw_grouped_gemm(const void* a, int a_dtype, const int32_t* place_
 #define FW_GG_LAUNCH(TA, TW, TO)                                                                                                   \
     {                                                                                                                              \
         if (gated) grouped_gemm_kernel<TA, TW, TO, true><<<grid, 256, 0, s>>>((const TA*)a, place_row, (const TW*)w, expert_begin, \
-                                                                              (TO*)out, experts, N, K);                           \
+                                                                              (TO*)out, experts, N, K, unit);                     \
         else grouped_gemm_kernel<TA, TW, TO, false><<<grid, 256, 0, s>>>((const TA*)a, place_row, (const TW*)w, expert_begin,      \
-                                                                         (TO*)out, experts, N, K);                                \
+                                                                         (TO*)out, experts, N, K, unit);                          \
     }
     if (a_dtype == FW_F32 && w_dtype == FW_F32 && out_dtype == FW_F32) FW_GG_LAUNCH(float, float, float)
     else if (a_dtype == FW_BF16 && w_dtype == FW_BF16 && out_dtype == FW_BF16) FW_GG_LAUNCH(bf16_t, bf16_t, bf16_t)

@@ -20,7 +20,7 @@ F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256          # of the matrix-core attention kernels
 MAX_PLAIN_HEAD_DIM = 512    # of the plain attention kernels, which serve what the others do not take
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _lib = None
 
@@ -290,6 +290,15 @@ def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor):
     return cos, sin
 
 
+def query_temperature(positions: torch.Tensor, coef: float, every: int) -> torch.Tensor:
+    """float32 [rows]: 1 + coef * ln(floor((position + 1) / every) + 1)."""
+    _dev(positions)
+    _want(positions, torch.int32, "positions")
+    out = torch.empty((positions.numel(),), dtype=torch.float32, device=positions.device)
+    _check(library().fw_query_temperature(_p(positions), _p(out), positions.numel(), ctypes.c_float(coef), int(every), _stream()))
+    return out
+
+
 def shortconv(bcx: torch.Tensor, taps: torch.Tensor, conv_bias: Optional[torch.Tensor], state: torch.Tensor,
               row_seg: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int,
               out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -340,8 +349,10 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
                           cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rotary_dim: int,
                           k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                           row_seg: torch.Tensor, row_pos: torch.Tensor, write_kv: bool = True,
-                          v_dim: Optional[int] = None, interleaved: bool = False, q_only: bool = False) -> torch.Tensor:
+                          v_dim: Optional[int] = None, interleaved: bool = False, q_only: bool = False,
+                          q_row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The output and the cache take the pages' dtype; ``qkv`` may be float32 beside bfloat16 pages.
+    ``q_row_scale`` (float32 [rows]): a factor on each row's finished queries.
     ``v_dim``: the size of a value head where it is not ``head_dim``. ``interleaved``: channel 2i turns
     with channel 2i + 1 instead of channel i with channel i + rotary_dim / 2."""
     _dev(qkv, q_norm_weight, k_norm_weight, cos, sin, k_pages, v_pages, block_table, row_seg, row_pos)
@@ -367,16 +378,32 @@ def qk_norm_rope_kv_write(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, 
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("qk_norm_rope: batch index arrays are too short")
     q_out = torch.empty((rows, num_heads * head_dim), dtype=k_pages.dtype, device=qkv.device)
+    _row_scale(q_row_scale, rows)
     _check(library().fw_qk_norm_rope_kv_write(
         _p(qkv), _code(qkv.dtype), _p(q_out), _code(k_pages.dtype), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin),
         rotary_dim, _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg), _p(row_pos), rows,
-        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), int(interleaved), int(q_only), _stream()))
+        num_heads, num_kv_heads, head_dim, v_dim, PAGE_SIZE, pages, int(write_kv), int(interleaved), int(q_only), _p(q_row_scale), _stream()))
     return q_out
 
 
-def _sinks(sinks: Optional[torch.Tensor], num_heads: int, keep_first: int, window: int, chunk: int):
+def _row_scale(q_row_scale: Optional[torch.Tensor], rows: int) -> None:
+    if q_row_scale is not None:
+        _dev(q_row_scale)
+        _want(q_row_scale, torch.float32, "q_row_scale")
+        if q_row_scale.numel() < rows:
+            raise KernelError(f"a factor per row: {q_row_scale.numel()} for {rows} rows")
+
+
+def _sinks(sinks: Optional[torch.Tensor], num_heads: int, keep_first: int, window: int, chunk: int,
+           slopes: Optional[torch.Tensor] = None):
     """Checks what the mask and the softmax take beyond a window: ``keep_first`` first keys that stay seen
-    (beside a window only) and one more term exp(sinks[head]) in the denominator (float32 [heads])."""
+    (beside a window only), one more term exp(sinks[head]) in the denominator (float32 [heads]) and a bias by
+    distance (``slopes`` float32 [heads]: slopes[head] * (row's position - key's position) is taken off a score)."""
+    if slopes is not None:
+        _dev(slopes)
+        _want(slopes, torch.float32, "slopes")
+        if slopes.shape != (num_heads,):
+            raise KernelError(f"attention: slopes are {tuple(slopes.shape)}, expected one per head ({num_heads})")
     if keep_first < 0 or (keep_first and chunk):
         raise KernelError(f"attention: {keep_first} first keys are kept beside a window, not beside chunks")
     if sinks is not None:
@@ -384,13 +411,14 @@ def _sinks(sinks: Optional[torch.Tensor], num_heads: int, keep_first: int, windo
         _want(sinks, torch.float32, "sinks")
         if sinks.shape != (num_heads,):
             raise KernelError(f"attention: sinks are {tuple(sinks.shape)}, expected one per head ({num_heads})")
-    return int(keep_first) if window else 0, _p(sinks)
+    return int(keep_first) if window else 0, _p(sinks), _p(slopes)
 
 
 def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, k_pages: torch.Tensor,
                       v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                       scale: float, window: int = 0, v_dim: Optional[int] = None, chunk: int = 0,
-                      softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``v_dim``: the size of a value head (and of a head's output) where it is not ``head_dim``.
     ``chunk`` > 0: a row sees only the keys of its own chunk of that many positions; ``softcap`` c > 0:
     score <- c tanh(score / c)."""
@@ -409,7 +437,7 @@ def attention_generic(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(library().fw_attention_generic(
         _p(q), _p(out), _code(q.dtype), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(row_seg),
         _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window), int(chunk),
-        ctypes.c_float(softcap), *_sinks(sinks, num_heads, keep_first, window, chunk), PAGE_SIZE, pages, _stream()))
+        ctypes.c_float(softcap), *_sinks(sinks, num_heads, keep_first, window, chunk, slopes), PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -916,7 +944,8 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
                       v_pages: torch.Tensor, block_table: torch.Tensor, tile_seg: torch.Tensor, tile_row0: torch.Tensor,
                       seg_row0: torch.Tensor, row_pos: torch.Tensor, scale: float, window: int = 0,
                       heads_together: int = 0, out: Optional[torch.Tensor] = None, v_dim: Optional[int] = None,
-                      chunk: int = 0, softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      chunk: int = 0, softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``heads_together``: query heads of a kv group per workgroup (1, or 4 up to head_dim 64), 0: the
     kernel's choice. Only the rows of the given tiles are written (into ``out`` if given)."""
     _dev(q, k_pages, v_pages, block_table, tile_seg, tile_row0, seg_row0, row_pos)
@@ -938,7 +967,7 @@ def attention_prefill(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_d
     _check(library().fw_attention_prefill(
         _p(q), _p(out), _p(k_pages), _p(v_pages), _p(block_table), block_table.shape[1], _p(tile_seg), _p(tile_row0),
         tile_seg.numel(), _p(seg_row0), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
-        int(window), int(chunk), ctypes.c_float(softcap), *_sinks(sinks, num_heads, keep_first, window, chunk), PAGE_SIZE, pages,
+        int(window), int(chunk), ctypes.c_float(softcap), *_sinks(sinks, num_heads, keep_first, window, chunk, slopes), PAGE_SIZE, pages,
         int(heads_together), _stream()))
     return out
 
@@ -956,7 +985,8 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
                      v_pages: torch.Tensor, block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor,
                      scale: float, max_context: int, window: int = 0, out: Optional[torch.Tensor] = None,
                      decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
-                     softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One row per request; ``max_context`` bounds position + 1 of every row (the host knows it).
     ``decode_work``: one int32 on the device, the runs of 4 pages that the rows see together (the
     sum of ceil((position + 1) / 256)): the kernel shares the work out by it (fewer, longer
@@ -972,7 +1002,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    keep_first, sinks_at = _sinks(sinks, num_heads, keep_first, window, chunk)
+    keep_first, sinks_at, slopes_at = _sinks(sinks, num_heads, keep_first, window, chunk, slopes)
     splits = decode_splits(max_context, window, chunk, keep_first)
     partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=q.device)
     if out is None:
@@ -985,7 +1015,7 @@ def attention_decode(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_di
         _p(q), _p(out), _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages),
         _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale),
-        int(window), int(chunk), ctypes.c_float(softcap), keep_first, sinks_at, PAGE_SIZE, pages, _stream()))
+        int(window), int(chunk), ctypes.c_float(softcap), keep_first, sinks_at, slopes_at, PAGE_SIZE, pages, _stream()))
     return out
 
 
@@ -996,7 +1026,8 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
                            scale: float, max_context: int, window: int = 0, write_kv: bool = True,
                            decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
                            softcap: float = 0.0, interleaved: bool = False, q_only: bool = False, keep_first: int = 0,
-                           sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           sinks: Optional[torch.Tensor] = None, slopes: Optional[torch.Tensor] = None,
+                           q_row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One row per request, from the step's raw projections ``qkv`` (float32 [rows, (heads + 2 kv
     heads) * head_dim]): per-head norm and rotation of queries and keys, the new keys and values
     into their pages, and the split-key attention, in one kernel. Returns bfloat16 [rows, heads *
@@ -1023,17 +1054,19 @@ def attention_decode_fused(qkv: torch.Tensor, num_heads: int, num_kv_heads: int,
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("attention: batch index arrays are too short")
-    keep_first, sinks_at = _sinks(sinks, num_heads, keep_first, window, chunk)
+    keep_first, sinks_at, slopes_at = _sinks(sinks, num_heads, keep_first, window, chunk, slopes)
     splits = decode_splits(max_context, window, chunk, keep_first)
     partial = torch.empty((rows, num_heads, splits, v_dim + 4), dtype=torch.float32, device=qkv.device)
     out = torch.empty((rows, num_heads * v_dim), dtype=torch.bfloat16, device=qkv.device)
     group = num_heads // num_kv_heads
     tickets = _medium_counters(qkv.device, rows * num_kv_heads * ((group + 15) // 16))
+    _row_scale(q_row_scale, rows)
     _check(library().fw_attention_decode_fused(
         _p(qkv), _p(q_norm_weight), _p(k_norm_weight), ctypes.c_float(eps), _p(cos), _p(sin), int(rotary_dim), int(write_kv), _p(out),
         _p(partial), splits, int(max_context), _work(decode_work), _p(tickets), tickets.numel(), _p(k_pages), _p(v_pages), _p(block_table),
         block_table.shape[1], _p(row_seg), _p(row_pos), rows, num_heads, num_kv_heads, head_dim, v_dim, ctypes.c_float(scale), int(window),
-        int(chunk), ctypes.c_float(softcap), int(interleaved), int(q_only), keep_first, sinks_at, PAGE_SIZE, pages, _stream()))
+        int(chunk), ctypes.c_float(softcap), int(interleaved), int(q_only), keep_first, sinks_at, slopes_at, _p(q_row_scale), PAGE_SIZE, pages,
+        _stream()))
     return out
 
 
@@ -1047,7 +1080,8 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
               v_pages: torch.Tensor, block_table: torch.Tensor, ctx, scale: float, window: int = 0,
               tile_seg: Optional[torch.Tensor] = None, tile_row0: Optional[torch.Tensor] = None,
               decode_work: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: int = 0,
-              softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+              softcap: float = 0.0, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                      slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """bfloat16 with a head size in steps of 16 runs on the matrix cores: the split-key decode
     kernel for segments of one row (all of them, or those a mixed step begins with: a single row
     would hold a 64-row tile of the prompt kernel and walk its whole context alone), the tiled
@@ -1060,7 +1094,7 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
     if fast and ctx.all_decode:
         return attention_decode(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                                 ctx.row_pos, scale, ctx.max_context, window, decode_work=decode_work, v_dim=v_dim,
-                                chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
+                                chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks, slopes=slopes)
     if fast:
         if tile_seg is None or tile_row0 is None:
             raise KernelError("attention: the tiled kernel needs the step's query tiles")
@@ -1074,17 +1108,17 @@ def attention(q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
         if single == 0:
             return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, tile_seg,
                                      tile_row0, ctx.seg_row0, ctx.row_pos, scale, window, heads_together=together, v_dim=v_dim,
-                                     chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
+                                     chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks, slopes=slopes)
         out = torch.empty((q.shape[0], num_heads * v_dim), dtype=q.dtype, device=q.device)
         attention_decode(q[:single], num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
                          ctx.row_pos, scale, ctx.max_context, window, out=out[:single], decode_work=decode_work, v_dim=v_dim,
-                         chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
+                         chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks, slopes=slopes)
         return attention_prefill(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table,
                                  tile_seg[single:], tile_row0[single:], ctx.seg_row0, ctx.row_pos, scale, window,
                                  heads_together=together, out=out, v_dim=v_dim, chunk=chunk, softcap=softcap,
-                                 keep_first=keep_first, sinks=sinks)
+                                 keep_first=keep_first, sinks=sinks, slopes=slopes)
     return attention_generic(q, num_heads, num_kv_heads, head_dim, k_pages, v_pages, block_table, ctx.row_seg,
-                             ctx.row_pos, scale, window, v_dim=v_dim, chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks)
+                             ctx.row_pos, scale, window, v_dim=v_dim, chunk=chunk, softcap=softcap, keep_first=keep_first, sinks=sinks, slopes=slopes)
 
 
 # ---- the gated delta rule -----------------------------------------------------------------------------
@@ -1293,47 +1327,85 @@ def gelu_gate_rows(z: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, col0
 
 # ---- attention over a cached latent ------------------------------------------------------------------------
 def latent_norm_write(raw: torch.Tensor, weight: torch.Tensor, eps: float, k_pages: torch.Tensor, v_pages: torch.Tensor,
-                      block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor) -> None:
-    """The step's latents ``raw`` (float32 [rows, rank]; a view of some columns of wider rows will do), RMS-normed
-    times ``weight``, stored at each row's position in a cache of one key/value head of ``rank`` channels."""
-    _dev(weight, k_pages, v_pages, block_table, row_seg, row_pos)
+                      block_table: torch.Tensor, row_seg: torch.Tensor, row_pos: torch.Tensor, rot: int = 0,
+                      cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, turn: Optional[int] = None) -> None:
+    """The step's latents ``raw`` (float32 [rows, rank + rot]; a view of some columns of wider rows will do): the first
+    rank columns RMS-normed times ``weight`` and stored at each row's position in a cache of one key/value head; the last
+    ``rot`` columns (a key part all heads share) turned by the row's angles (neighbouring channels paired; ``cos``, ``sin``
+    float32 [rows, rot / 2]) and stored behind the latent in the keys' layout, whose head then has rank + rot channels."""
+    _dev(weight, k_pages, v_pages, block_table, row_seg, row_pos, cos, sin)
     _dev_rows(raw, "raw")
     _want(raw, torch.float32, "raw")
     _want(weight, torch.float32, "weight")
-    rows, rank = raw.shape
+    rows, rank = raw.shape[0], raw.shape[1] - int(rot)
     if weight.shape != (rank,):
         raise KernelError(f"latent_norm_write: weight is {tuple(weight.shape)}, the latent has {rank} channels")
-    pages = _check_pages(k_pages, v_pages, 1, rank, k_pages.dtype, rank)
+    turn = int(rot) if turn is None else int(turn)      # the first so many channels of the part are turned, the rest pass
+    if turn:
+        for t in (cos, sin):
+            if t is None or t.dtype != torch.float32 or t.shape != (rows, turn // 2):
+                raise KernelError(f"latent_norm_write: {turn} turned channels need float32 tables {(rows, turn // 2)}")
+    pages = _check_pages(k_pages, v_pages, 1, rank + int(rot), k_pages.dtype, rank)
     for name, t in (("block_table", block_table), ("row_seg", row_seg), ("row_pos", row_pos)):
         _want(t, torch.int32, name)
     if block_table.dim() != 2 or row_seg.numel() < rows or row_pos.numel() < rows:
         raise KernelError("latent_norm_write: batch index arrays are too short")
-    _check(library().fw_latent_norm_write(_p(raw), raw.stride(0) if rows > 1 else max(rank, raw.stride(0)), 0, _p(weight), ctypes.c_float(eps),
-                                          _p(k_pages), _p(v_pages), _code(k_pages.dtype), _p(block_table), block_table.shape[1],
-                                          _p(row_seg), _p(row_pos), rows, rank, PAGE_SIZE, pages, _stream()))
+    _check(library().fw_latent_norm_write(_p(raw), raw.stride(0) if rows > 1 else max(rank + int(rot), raw.stride(0)), 0, _p(weight),
+                                          ctypes.c_float(eps), _p(k_pages), _p(v_pages), _code(k_pages.dtype), _p(block_table),
+                                          block_table.shape[1], _p(row_seg), _p(row_pos), rows, rank, int(rot), turn, _p(cos), _p(sin),
+                                          PAGE_SIZE, pages, _stream()))
 
 
-def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None,
+                in_head: Optional[int] = None, out: Optional[torch.Tensor] = None, out_head: Optional[int] = None) -> torch.Tensor:
     """A map per head: ``x`` [rows, heads K] (rows may lie apart), ``w`` [heads, N, K] -> [rows, heads N], with
-    ``gate`` (float32 [rows, heads N], rows may lie apart) times its sigmoid."""
+    ``gate`` (float32 [rows, heads N], rows may lie apart) times its sigmoid. ``in_head``: a head's vector in ``x`` holds
+    that many channels of which the map reads the first K; ``out`` with ``out_head``: the results go to the first N
+    channels of each head's vector of ``out_head`` channels in the rows of ``out``."""
     _dev(w)
     _dev_rows(x, "x")
     heads, N, K = w.shape
     rows = x.shape[0]
-    if x.shape[1] != heads * K:
-        raise KernelError(f"head_linear: x is {tuple(x.shape)}, the weight {tuple(w.shape)}")
+    in_head = K if in_head is None else int(in_head)
+    if x.shape[1] != heads * in_head or in_head < K:
+        raise KernelError(f"head_linear: x is {tuple(x.shape)}, the weight {tuple(w.shape)}, a head's vector {in_head}")
     if gate is not None:
         _dev_rows(gate, "gate")
         if gate.shape != (rows, heads * N) or gate.dtype != torch.float32:
             raise KernelError(f"head_linear: the gate is {tuple(gate.shape)} {gate.dtype}, expected {(rows, heads * N)} float32")
-    out = torch.empty((rows, heads * N), dtype=out_dtype, device=x.device)
+    out_head = N if out_head is None else int(out_head)
+    if out is None:
+        out = torch.empty((rows, heads * out_head), dtype=out_dtype, device=x.device)
+    elif out.shape != (rows, heads * out_head) or out.dtype != out_dtype or not out.is_contiguous() or not out.is_cuda:
+        raise KernelError(f"head_linear: out is {tuple(out.shape)} {out.dtype}, expected {(rows, heads * out_head)} {out_dtype}")
+    if out_head < N or (gate is not None and out_head != N):
+        raise KernelError("head_linear: a head's outputs do not fit its vector (a gate goes with outputs side by side)")
 
     def stride(t: torch.Tensor, width: int) -> int:
         return t.stride(0) if rows > 1 else max(width, t.stride(0))
 
-    _check(library().fw_head_linear(_p(x), _code(x.dtype), stride(x, heads * K), _p(w), _code(w.dtype), _p(gate),
+    _check(library().fw_head_linear(_p(x), _code(x.dtype), stride(x, heads * in_head), _p(w), _code(w.dtype), _p(gate),
                                     stride(gate, heads * N) if gate is not None else 0, _p(out), _code(out_dtype), rows, heads, N, K,
-                                    _stream()))
+                                    in_head, out_head, heads * out_head, _stream()))
+    return out
+
+
+def rotate_place(x: torch.Tensor, heads: int, col0: int, rot: int, cos: torch.Tensor, sin: torch.Tensor, out: torch.Tensor,
+                 out_col0: int, turn: Optional[int] = None) -> torch.Tensor:
+    """Channels col0 .. col0 + rot - 1 of every head's vector in ``x`` [rows, heads * in_head], neighbouring channels
+    turned by the row's angles (``cos``, ``sin`` float32 [rows, rot / 2]), stored from channel ``out_col0`` of the head's
+    vector in ``out`` [rows, heads * out_head]."""
+    _dev(x, cos, sin, out)
+    rows = x.shape[0]
+    if x.dim() != 2 or out.dim() != 2 or x.shape[1] % heads or out.shape[1] % heads or out.shape[0] != rows:
+        raise KernelError(f"rotate_place: {tuple(x.shape)} -> {tuple(out.shape)} with {heads} heads")
+    turn = int(rot) if turn is None else int(turn)      # the first so many channels are turned, the rest pass
+    for t in ((cos, sin) if turn else ()):
+        if t is None or t.dtype != torch.float32 or t.shape != (rows, turn // 2):
+            raise KernelError(f"rotate_place: {turn} turned channels need float32 tables {(rows, turn // 2)}")
+    _check(library().fw_rotate_place(_p(x), _code(x.dtype), x.shape[1], x.shape[1] // heads, int(col0), _p(cos), _p(sin), _p(out),
+                                     _code(out.dtype), out.shape[1], out.shape[1] // heads, int(out_col0), rows, heads, int(rot), turn,
+                                     _stream()))
     return out
 
 
@@ -1409,9 +1481,12 @@ def wkv_recurrence(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, a: torch.T
 
 
 # ---- a mixture of feed-forward units chosen per token ------------------------------------------------------------
-def moe_route(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int):
+def moe_route(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int, groups: int = 1, keep: int = 1,
+              score_all: bool = False):
     """(chosen int32 [rows, top], weight float32 [rows, top]): the ``top`` largest of logits + bias per row, largest
-    first (ties: the lowest id), and the softmax over those alone."""
+    first (ties: the lowest id), and the softmax over those alone. ``groups`` > 1: only experts of the ``keep`` groups
+    (of neighbours, equal in size) whose best expert scores highest can be chosen. ``score_all``: the weights are the
+    softmax over all experts at the chosen ones, divided by their sum + 1e-20."""
     _dev(logits, bias)
     _want(logits, torch.float32, "logits")
     rows, experts = logits.shape
@@ -1419,7 +1494,8 @@ def moe_route(logits: torch.Tensor, bias: Optional[torch.Tensor], top: int):
         raise KernelError("moe_route: the bias is float32 [experts]")
     chosen = torch.empty((rows, top), dtype=torch.int32, device=logits.device)
     weight = torch.empty((rows, top), dtype=torch.float32, device=logits.device)
-    _check(library().fw_moe_route(_p(logits), _p(bias), _p(chosen), _p(weight), rows, experts, int(top), _stream()))
+    _check(library().fw_moe_route(_p(logits), _p(bias), _p(chosen), _p(weight), rows, experts, int(top), int(groups), int(keep),
+                                  int(score_all), _stream()))
     return chosen, weight
 
 
@@ -1437,9 +1513,10 @@ def moe_arrange(chosen: torch.Tensor, experts: int):
 
 
 def grouped_gemm(a: torch.Tensor, place_row: Optional[torch.Tensor], w: torch.Tensor, expert_begin: torch.Tensor, places: int,
-                 gated: bool, out_dtype: torch.dtype) -> torch.Tensor:
+                 gated: bool, out_dtype: torch.dtype, glu: Optional[tuple] = None) -> torch.Tensor:
     """out[place] = a[place_row[place]] . w[expert of place]^T (``place_row`` None: a[place]); ``w`` [experts, N, K], or
-    with ``gated`` [experts, 2 N, K] (gate rows, then up rows) and out = silu(gate) * up. Returns [places, N]."""
+    with ``gated`` [experts, 2 N, K] (gate rows, then up rows) and out = silu(gate) * up, or with ``glu`` = (limit, alpha,
+    shift) the unit with clamped halves. Returns [places, N]."""
     _dev(a, place_row, w, expert_begin)
     experts, n_rows, K = w.shape
     N = n_rows // 2 if gated else n_rows
@@ -1454,7 +1531,7 @@ def grouped_gemm(a: torch.Tensor, place_row: Optional[torch.Tensor], w: torch.Te
         raise KernelError("grouped_gemm: fewer rows than places")
     out = torch.empty((places, N), dtype=out_dtype, device=a.device)
     _check(library().fw_grouped_gemm(_p(a), _code(a.dtype), _p(place_row), _p(w), _code(w.dtype), _p(expert_begin), _p(out),
-                                     _code(out_dtype), int(gated), int(places), experts, N, K, _stream()))
+                                     _code(out_dtype), int(gated), int(places), experts, N, K, *_glu(glu if gated else None), _stream()))
     return out
 
 
@@ -1470,3 +1547,69 @@ def moe_combine_(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, pair_pl
         raise KernelError(f"moe_combine: x {tuple(x.shape)}, y {tuple(y.shape)}, weight {tuple(weight.shape)}, places {tuple(pair_place.shape)}")
     _check(library().fw_moe_combine(_p(x), _p(y), _p(weight), _p(pair_place), rows, top, hidden, _stream()))
     return x
+
+
+# ---- a short causal convolution per channel, and a gated linear recurrence per channel ---------------------------------
+def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, row_seg: torch.Tensor,
+                seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int, single_rows: bool = False,
+                echo: Optional[tuple] = None) -> torch.Tensor:
+    """y[t, c] = sum_j taps[c, j] * x[t - L + 1 + j, c] (+ bias[c]) over the step's segments, float32. ``x`` float32
+    [rows, channels] (rows may lie apart), ``taps`` [channels, L] with the last column the current token's, ``state``
+    float32 [slots, channels, L - 1]: the inputs before each segment's first row, read and moved on. ``echo`` = (first
+    channel, count): those channels are written once more behind the others (the output is then that much wider).
+    ``single_rows``: every segment is one row."""
+    _dev(taps, bias, state, row_seg, seg_row0, seg_slot)
+    _dev_rows(x, "x")
+    for name, t in (("x", x), ("taps", taps), ("state", state)):
+        _want(t, torch.float32, name)
+    rows, channels = x.shape
+    L = taps.shape[1]
+    if taps.shape != (channels, L) or state.dim() != 3 or state.shape[1:] != (channels, L - 1):
+        raise KernelError(f"causal_conv: x {tuple(x.shape)}, taps {tuple(taps.shape)}, state {tuple(state.shape)}")
+    if bias is not None and (bias.dtype != torch.float32 or bias.shape != (channels,)):
+        raise KernelError("causal_conv: the bias is float32 [channels]")
+    for name, t, n in (("row_seg", row_seg, rows), ("seg_row0", seg_row0, segments + 1), ("seg_slot", seg_slot, segments)):
+        _want(t, torch.int32, name)
+        if t.numel() < n:
+            raise KernelError(f"causal_conv: {name} holds {t.numel()} entries, needs {n}")
+    first, count = echo if echo is not None else (0, 0)
+    if count and not (0 <= first and first + count <= channels):
+        raise KernelError(f"causal_conv: channels {first}..{first + count} of {channels}")
+    out = torch.empty((rows, channels + count), dtype=torch.float32, device=x.device)
+    stride = x.stride(0) if rows > 1 else max(channels, x.stride(0))
+    _check(library().fw_causal_conv(_p(x), stride, _p(taps), _p(bias), _p(state), _p(row_seg), _p(seg_row0), _p(seg_slot), _p(out),
+                                    channels + count, int(first), int(count), channels, rows, int(segments), channels, L,
+                                    state.shape[0], int(bool(single_rows)), _stream()))
+    return out
+
+
+def rglru_scan(u: torch.Tensor, gates: torch.Tensor, y: torch.Tensor, r_bias: torch.Tensor, i_bias: torch.Tensor, lam: torch.Tensor,
+               rate: float, state: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int, block_width: int,
+               out_dtype: torch.dtype) -> torch.Tensor:
+    """The gated linear recurrence per channel over the step's segments: r = sigmoid(g_r + r_bias), i = sigmoid(g_i +
+    i_bias), a = exp(-rate r softplus(lam)), S <- a S + sqrt(1 - a^2) i u, out = S * gelu_tanh(y). ``u``, ``y`` float32
+    [rows, channels] (rows may lie apart); ``gates`` float32 [rows, 2 channels], block after block [g_r of the block | g_i
+    of the block]; ``state`` float32 [slots, channels], read and moved on."""
+    _dev(gates, r_bias, i_bias, lam, state, seg_row0, seg_slot)
+    _dev_rows(u, "u")
+    _dev_rows(y, "y")
+    rows, channels = u.shape
+    for name, t in (("u", u), ("gates", gates), ("y", y), ("r_bias", r_bias), ("i_bias", i_bias), ("lam", lam), ("state", state)):
+        _want(t, torch.float32, name)
+    if y.shape != (rows, channels) or gates.shape != (rows, 2 * channels) or channels % block_width or state.dim() != 2 \
+            or state.shape[1] != channels or any(t.numel() != channels for t in (r_bias, i_bias, lam)):
+        raise KernelError(f"rglru_scan: u {tuple(u.shape)}, gates {tuple(gates.shape)}, y {tuple(y.shape)}, state {tuple(state.shape)}, "
+                          f"blocks of {block_width}")
+    for name, t, n in (("seg_row0", seg_row0, segments + 1), ("seg_slot", seg_slot, segments)):
+        _want(t, torch.int32, name)
+        if t.numel() < n:
+            raise KernelError(f"rglru_scan: {name} holds {t.numel()} entries, needs {n}")
+    out = torch.empty((rows, channels), dtype=out_dtype, device=u.device)
+
+    def stride(t: torch.Tensor) -> int:
+        return t.stride(0) if rows > 1 else max(channels, t.stride(0))
+
+    _check(library().fw_rglru_scan(_p(u), stride(u), _p(gates), 2 * channels, _p(y), stride(y), _p(r_bias), _p(i_bias), _p(lam),
+                                   ctypes.c_float(rate), _p(state), _p(seg_row0), _p(seg_slot), _p(out), _code(out_dtype), rows,
+                                   int(segments), channels, int(block_width), state.shape[0], _stream()))
+    return out

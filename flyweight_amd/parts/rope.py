@@ -71,6 +71,24 @@ class RotaryInterleaved(RotaryNeox):
     interleaved = True
 
 
+@register_position_encoding("query_temperature")
+class QueryTemperature(PositionEncoding):
+    """No rotation: a factor per row on the finished queries, 1 + coef * ln(floor((p + 1) / every) + 1) at position p
+    (1 up to position every - 2, then a step up every ``every`` positions). ``tables`` gives float32 [rows]."""
+    graph_safe = True
+    rotary_dim = 0
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        self.coef = float(spec["coef"])
+        self.every = int(spec["every"])
+        if self.every < 1:
+            raise ConfigError(f"a query temperature steps every {self.every} positions (at least 1)")
+
+    def tables(self, ctx):
+        return ops.query_temperature(ctx.encoding_pos, self.coef, self.every)
+
+
 @register_position_encoding("none")
 class NoPosition(PositionEncoding):
     graph_safe = True
