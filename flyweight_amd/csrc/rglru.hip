@@ -167,8 +167,9 @@ __global__ __launch_bounds__(64) void rglru_scan_kernel(
 #pragma unroll
         for (int k = 0; k < SCAN_ROWS; ++k) {
             const float r = rglru_sigmoid(gr[k] + br), i = rglru_sigmoid(gi[k] + bi);
+            // 1 - a^2 as -expm1(2 log a): a channel that barely forgets has a near 1, where 1 - a * a would lose its digits
             a[k] = expf(decay * r);
-            b[k] = sqrtf(1.0f - a[k] * a[k]) * (i * uu[k]);
+            b[k] = sqrtf(-expm1f(2.0f * decay * r)) * (i * uu[k]);
             yy[k] = rglru_gelu_tanh(yy[k]);
         }
 #pragma unroll

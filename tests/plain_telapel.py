@@ -77,14 +77,20 @@ def rglru(h: np.ndarray, w: Dict[str, np.ndarray], blocks: int, state=None):
         part = u[:, b * size:(b + 1) * size]
         r[:, b * size:(b + 1) * size] = sigmoid(part @ w["ra"][b].T + w["ra.b"][b])
         i[:, b * size:(b + 1) * size] = sigmoid(part @ w["ri"][b].T + w["ri.b"][b])
-    a = np.exp(-8.0 * r * softplus(w["lam"]))
-    if S is None:
-        S = np.zeros(C)
+    out, S = gated_recurrence(u, r, i, w["lam"], S)
+    return (out * y) @ w["o"].T, (S, before)
+
+
+def gated_recurrence(u: np.ndarray, r: np.ndarray, i: np.ndarray, lam: np.ndarray, S: Optional[np.ndarray], rate: float = 8.0):
+    """a = exp(-rate r softplus(lam)); S_t = a_t S_(t-1) + sqrt(1 - a_t^2) i_t u_t, from S (zeros if None). Returns
+    every S_t [T, C] and the last one."""
+    a = np.exp(-rate * r * softplus(lam))
+    S = np.zeros(u.shape[1]) if S is None else S
     out = np.zeros_like(u)
-    for t in range(T):
+    for t in range(u.shape[0]):
         S = a[t] * S + np.sqrt(1.0 - a[t] ** 2) * i[t] * u[t]
         out[t] = S
-    return (out * y) @ w["o"].T, (S, before)
+    return out, S
 
 
 # ----- rotation of neighbouring channels ------------------------------------------------------------
@@ -144,21 +150,40 @@ def key_value_attention(h: np.ndarray, w: Dict[str, np.ndarray], sizes: Dict, ep
     values = np.concatenate([past_v, k.reshape(T, G, d)], axis=0)             # the keys before their norm
     keys = np.concatenate([past_k, rms_norm(k.reshape(T, G, d), w["k.norm"], eps)], axis=0)
     q = rms_norm(q.reshape(T, H, d), w["q.norm"], eps)
-    out = np.zeros((T, H, d))
+    for t in range(T):
+        q[t] *= query_factor(start + t, sizes["temp_coef"], sizes.get("temp_every"))
+    out = biased_heads(q, keys, values, start, sizes["scale"], sizes.get("window"), sizes.get("softcap"))
+    return out.reshape(T, H * d) @ w["o"].T, (values, keys, before_q, before_k)
+
+
+def query_factor(position: int, coef: float, every: Optional[int]) -> float:
+    """1 + coef ln(floor((p + 1) / every) + 1); 1 where the design has none."""
+    return 1.0 + coef * math.log(math.floor((position + 1) / every) + 1.0) if every else 1.0
+
+
+def biased_heads(q: np.ndarray, keys: np.ndarray, values: np.ndarray, start: int, scale: float, window: Optional[int],
+                 softcap: Optional[float], exponent: float = 8.0) -> np.ndarray:
+    """q [T, H, d] are the rows at positions start .. start + T - 1 of a sequence whose keys [N, G, d] and values
+    [N, G, dv] are given from position 0 on. score = q . k * scale, capped (cap tanh(score / cap)), less slope_h *
+    distance with slope_h = 2^(-exponent (h + 1) / H); row i sees keys j with 0 <= i - j < window; the weights are
+    e^s / (1 + sum e^s). Returns [T, H, dv]."""
+    T, H, _ = q.shape
+    G = keys.shape[1]
+    out = np.zeros((T, H, values.shape[2]))
     for t in range(T):
         p = start + t
-        factor = 1.0 + sizes["temp_coef"] * math.log(math.floor((p + 1) / sizes["temp_every"]) + 1.0) if sizes.get("temp_every") else 1.0
-        first = 0 if sizes.get("window") is None else max(0, p - sizes["window"] + 1)
+        first = 0 if window is None else max(0, p - window + 1)
         js = np.arange(first, p + 1)
         for head in range(H):
             g = head // (H // G)
-            s = (keys[first:p + 1, g] @ (q[t, head] * factor)) * sizes["scale"]
-            if sizes.get("softcap"):
-                s = sizes["softcap"] * np.tanh(s / sizes["softcap"])
-            s = s - 2.0 ** (-8.0 * (head + 1) / H) * (p - js)
-            e = np.exp(s)
-            out[t, head] = (e / (1.0 + e.sum())) @ values[first:p + 1, g]
-    return out.reshape(T, H * d) @ w["o"].T, (values, keys, before_q, before_k)
+            s = (keys[first:p + 1, g] @ q[t, head]) * scale
+            if softcap:
+                s = softcap * np.tanh(s / softcap)
+            s = s - 2.0 ** (-exponent * (head + 1) / H) * (p - js)
+            top = max(s.max(), 0.0)
+            e = np.exp(s - top)
+            out[t, head] = (e / (np.exp(-top) + e.sum())) @ values[first:p + 1, g]
+    return out
 
 
 # ----- the feed-forward -------------------------------------------------------------------------
@@ -185,6 +210,27 @@ def route(h: np.ndarray, router: np.ndarray, top: int, groups: int, keep: int) -
         chosen[t] = np.argsort(-allowed, kind="stable")[:top]
         weight[t] = s[t, chosen[t]] / (s[t, chosen[t]].sum() + 1e-20)
     return chosen, weight
+
+
+def route_margin(h: np.ndarray, router: np.ndarray, top: int, groups: int, keep: int) -> np.ndarray:
+    """How clear each row's choice is, [T]: the smallest gap between what is chosen and what is not (the last kept
+    group's best logit against the first group left out, the last chosen expert's logit against the first one left
+    out), as a fraction of the row's largest logit in size. Rows near 0 are close calls: a rounding of h can turn them."""
+    z = h @ router.T
+    T, E = z.shape
+    margin = np.full(T, np.inf)
+    for t in range(T):
+        allowed = z[t].copy()
+        if groups > 1 and keep < groups:
+            best = np.sort(z[t].reshape(groups, E // groups).max(axis=1))[::-1]
+            margin[t] = best[keep - 1] - best[keep]
+            kept = np.argsort(-z[t].reshape(groups, E // groups).max(axis=1), kind="stable")[:keep]
+            allowed = np.concatenate([z[t, g * (E // groups):(g + 1) * (E // groups)] for g in kept])
+        if top < allowed.size:
+            ordered = np.sort(allowed)[::-1]
+            margin[t] = min(margin[t], ordered[top - 1] - ordered[top])
+        margin[t] /= max(np.abs(z[t]).max(), 1e-30)
+    return margin
 
 
 def mixture(h: np.ndarray, w: Dict[str, np.ndarray], sizes: Dict) -> np.ndarray:
@@ -236,9 +282,9 @@ class PlainTelapel:
     def start(self) -> List:
         return [None] * len(self.config["layers"])
 
-    def forward(self, tokens, states: Optional[List] = None, keep_layers: bool = False):
+    def forward(self, tokens, states: Optional[List] = None, keep_layers: bool = False, margins: Optional[List] = None):
         """Logits [T, vocab] of the next ``tokens`` of one sequence; ``states`` (from ``start`` or an earlier
-        call) is brought up to date in place."""
+        call) is brought up to date in place. ``margins``: a list that receives every mixture's ``route_margin``."""
         if states is None:
             states = self.start()
         x = self.tensors["embed"][np.asarray(tokens, dtype=np.int64)]
@@ -255,7 +301,100 @@ class PlainTelapel:
                 y, states[index] = key_value_attention(x, mix, _mixer_sizes(entry), self.eps, states[index])
             x = x + rms_norm(y, w["norm1"], self.eps)
             if entry.get("mlp") is not None:
+                if margins is not None:
+                    sizes = _ff_sizes(entry["mlp"])
+                    margins.append(route_margin(x, w["mlp.router"], sizes["top"], sizes["groups"], sizes["keep"]))
                 x = x + rms_norm(mixture(x, _under(w, "mlp."), _ff_sizes(entry["mlp"])), w["norm2"], self.eps)
             after.append(x.copy())
         logits = rms_norm(x, self.tensors["final.norm"], self.eps) @ self.tensors["embed"].T
         return (logits, after) if keep_layers else logits
+
+
+def forward(config: Dict, weights: Dict[str, np.ndarray], tokens) -> np.ndarray:
+    """Logits [T, vocab] of a whole sequence."""
+    return PlainTelapel(config, weights).forward(list(tokens))
+
+
+def greedy(config: Dict, weights: Dict[str, np.ndarray], prompt: List[int], new: int) -> List[int]:
+    """The prompt once, then token by token on the carried states."""
+    model = PlainTelapel(config, weights)
+    states = model.start()
+    logits = model.forward(list(prompt), states)
+    out = []
+    for _ in range(new):
+        out.append(int(np.argmax(logits[-1])))
+        logits = model.forward([out[-1]], states)
+    return out
+
+
+# ----- tensors of a model --------------------------------------------------------------------------------
+def tensor_shapes(config: Dict) -> Dict[str, Tuple[int, ...]]:
+    D, V = config["width"], config["vocab"]
+    shapes: Dict[str, Tuple[int, ...]] = {"embed": (V, D), "final.norm": (D,)}
+    for index, layer in enumerate(config["layers"]):
+        if layer.get("weights_of") is not None:
+            continue
+        base, m = f"l{index}.", layer["mixer"]
+        shapes[base + "norm1"] = (D,)
+        mix = base + "mix."
+        if layer["type"] == "rglru":
+            C, B, L = m["width"], m["blocks"], m["conv"]
+            shapes.update({mix + "y": (C, D), mix + "y.b": (C,), mix + "x": (C, D), mix + "x.b": (C,), mix + "conv": (C, L),
+                           mix + "conv.b": (C,), mix + "ra": (B, C // B, C // B), mix + "ra.b": (B, C // B),
+                           mix + "ri": (B, C // B, C // B), mix + "ri.b": (B, C // B), mix + "lam": (C,), mix + "o": (D, C)})
+        elif layer["type"] == "latent_attention":
+            H, d, dr, dv, rq, rk = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["q_rank"], m["kv_rank"]
+            shapes.update({mix + "dq": (rq, D), mix + "dq.norm": (rq,), mix + "uq": (H * (d + dr), rq), mix + "dkv": (rk + dr, D),
+                           mix + "dkv.norm": (rk,), mix + "uk": (H * d, rk), mix + "uv": (H * dv, rk), mix + "o": (D, H * dv)})
+        else:
+            H, G, d, L = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["conv"]
+            shapes.update({mix + "q": (H * d, D), mix + "q.b": (H * d,), mix + "k": (G * d, D), mix + "k.b": (G * d,),
+                           mix + "q.norm": (d,), mix + "k.norm": (d,), mix + "q.conv": (H * d, L), mix + "k.conv": (G * d, L),
+                           mix + "o": (D, H * d)})
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            shapes[base + "norm2"] = (D,)
+            ff = base + "mlp."
+            shapes[ff + "router"] = (mlp["router"]["experts"], D)
+            units = [(f"e{e}.", mlp["expert"]["ff"]) for e in range(mlp["router"]["experts"])]
+            if mlp.get("shared"):
+                units.append(("shared.", mlp["shared"]["ff"]))
+            for unit, width in units:
+                shapes.update({ff + unit + "gate": (width, D), ff + unit + "up": (width, D), ff + unit + "down": (D, width)})
+    return shapes
+
+
+def random_weights(config: Dict, seed: int, experts_alike: float = 0.75) -> Dict[str, np.ndarray]:
+    """Weights that make every part count: matrices keep the size of what passes through them (the router's and the
+    units' somewhat more, so that the clamps bite), decays from barely forgetting to forgetting at once, biases and
+    taps of visible size. The experts of a layer share ``experts_alike`` of their weights: where bfloat16 rounding turns
+    a close call of the router the output then moves by a part of an expert, not by all of it, while in float32 any
+    wrong choice still shows far above the comparison's limit."""
+    rng = np.random.default_rng(seed)
+    weights: Dict[str, np.ndarray] = {}
+    common: Dict[Tuple[str, str], np.ndarray] = {}
+    for name, shape in tensor_shapes(config).items():
+        leaf = name.split(".")[-1]
+        parts = name.split(".")
+        if len(parts) == 4 and parts[1] == "mlp" and parts[2].startswith("e") and experts_alike:
+            if (parts[0], leaf) not in common:
+                common[parts[0], leaf] = rng.normal(0.0, 1.5 if leaf != "down" else 1.0, shape) / math.sqrt(shape[-1])
+            own = rng.normal(0.0, 1.5 if leaf != "down" else 1.0, shape) / math.sqrt(shape[-1])
+            weights[name] = experts_alike * common[parts[0], leaf] + (1.0 - experts_alike) * own
+            continue
+        if leaf in ("norm1", "norm2", "norm") or name == "final.norm":
+            value = rng.uniform(0.6, 1.4, shape)
+        elif leaf == "lam":
+            value = rng.uniform(-5.0, 1.0, shape)
+        elif leaf == "b":
+            value = rng.normal(0.0, 0.5, shape)
+        elif leaf == "conv":
+            value = rng.normal(0.0, 0.6, shape)
+        elif name == "embed":
+            value = rng.normal(0.0, 1.0, shape)
+        elif leaf == "router" or leaf in ("gate", "up"):
+            value = rng.normal(0.0, 1.5, shape) / math.sqrt(shape[-1])
+        else:
+            value = rng.normal(0.0, 1.0, shape) / math.sqrt(shape[-1])
+        weights[name] = value
+    return weights
