@@ -156,6 +156,40 @@ def dalerax_configs(size: dict):
     return dalerax, koketar_configs(size)[0]
 
 
+# Telapel (layers of one mixer each: a gated linear recurrence per channel behind a short convolution, softmax attention
+# over a cached latent with a rotated key part, windowed attention whose values are its keys with convolutions on q and
+# k, a cap, a bias by distance and a query factor; every feed-forward a mixture of clamped units chosen among the best
+# groups of experts, with a shared unit; the last layer runs the first one's weights) at the two sizes of DALERAX_SIZES,
+# beside the engine's closest existing model: a Dalerax of the same width, depth, vocabulary, experts and windows.
+TELAPEL_SIZES = {
+    "w1024": dict(DALERAX_SIZES["w1024"], lru_width=1280, lru_blocks=5, q_rank=384, kv_rank=128, rot_dim=64, latent_dim=64,
+                  groups=4, keep=2, limit=7.0),
+    "w2048": dict(DALERAX_SIZES["w2048"], lru_width=2560, lru_blocks=10, q_rank=768, kv_rank=192, rot_dim=64, latent_dim=128,
+                  groups=4, keep=2, limit=7.0),
+}
+
+
+def telapel_configs(size: dict):
+    """(Telapel configuration, Dalerax configuration of equal size)."""
+    from flyweight_amd.config import config_from_dict
+    moe = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"], "groups": {"count": size["groups"], "keep": size["keep"]}},
+           "expert": {"ff": size["expert_ff"], "limit": size["limit"]}, "shared": {"ff": size["shared_ff"], "limit": size["limit"]}}
+    recurrence = {"type": "rglru", "mixer": {"width": size["lru_width"], "blocks": size["lru_blocks"], "conv": size["conv"]}, "mlp": moe}
+    latent = {"type": "latent_attention", "mlp": moe,
+              "mixer": {"heads": size["heads"], "dim": size["latent_dim"], "rot_dim": size["rot_dim"], "vdim": size["vdim"],
+                        "q_rank": size["q_rank"], "kv_rank": size["kv_rank"], "scale": (size["latent_dim"] + size["rot_dim"]) ** -0.5,
+                        "rot": {"base": 10000.0, "dims": size["rot_dim"]}}}
+    attention = {"type": "attention", "mlp": moe,
+                 "mixer": {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"], "conv": 3,
+                           "scale": size["dim"] ** -0.5, "softcap": 30.0, "mask": {"size": size["window"]},
+                           "q_temp": {"coef": 0.5, "every": 256}}}
+    kinds = [recurrence, latent, attention, dict(recurrence, weights_of=0)]
+    layers = [kinds[index % 4] if index % 4 != 3 else dict(recurrence, weights_of=index - 3) for index in range(size["layers"])]
+    telapel = config_from_dict({"architecture": "Telapel", "vocab": size["vocab"], "width": size["width"], "norm": {"eps": 1e-6},
+                                "layers": layers})
+    return telapel, dalerax_configs(size)[0]
+
+
 def kernel_times(torch, run) -> dict:
     """Entry point of the kernel library -> microseconds of GPU time per call, over one call of ``run``
     (launched kernel by kernel, every call bracketed by two events)."""
@@ -528,10 +562,11 @@ def main() -> int:
     parser.add_argument("--only", choices=("decode", "prefill"), help="run one phase and print no JSON (for profiling)")
     parser.add_argument("--drawn", action="store_true", help="with --only decode: the requests draw their tokens "
                         "(temperature 0.8, top_k 40, top_p 0.95, min_p 0.05) instead of taking the most likely one")
-    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar", "vavelorn", "dalerax"), default="headline",
+    parser.add_argument("--workload", choices=("headline",) + tuple(WORKLOADS) + ("koketar", "vavelorn", "dalerax", "telapel"), default="headline",
                         help="headline: the LFM2-1.2B decode and prefill figures; long-context, mixed: a whole serving run; "
                              "koketar: prefill and decode of Koketar beside LFM2 at equal sizes, kernel by kernel; "
-                             "vavelorn: the same of Vavelorn beside Koketar; dalerax: the same of Dalerax beside Koketar")
+                             "vavelorn: the same of Vavelorn beside Koketar; dalerax: the same of Dalerax beside Koketar; "
+                             "telapel: the same of Telapel beside Dalerax")
     parser.add_argument("--requests", type=int, help="requests of a serving workload (default: as the workload names)")
     args = parser.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -545,8 +580,11 @@ def main() -> int:
     from flyweight_amd import Model
     from flyweight_amd.config import config_from_dict
 
-    if args.workload in ("koketar", "vavelorn", "dalerax"):
-        if args.workload == "dalerax":
+    if args.workload in ("koketar", "vavelorn", "dalerax", "telapel"):
+        if args.workload == "telapel":
+            record = koketar_run(torch, args, families=("telapel", "dalerax"), sizes=TELAPEL_SIZES, configs_of=telapel_configs,
+                                 title="Telapel", beside="Telapel beside Dalerax at equal width, depth, vocabulary, experts and windows")
+        elif args.workload == "dalerax":
             record = koketar_run(torch, args, families=("dalerax", "koketar"), sizes=DALERAX_SIZES, configs_of=dalerax_configs,
                                  title="Dalerax", beside="Dalerax beside Koketar at equal width, depth, vocabulary and feed-forward "
                                                          "width a token runs through")

@@ -364,7 +364,7 @@ def tensor_shapes(config: Dict) -> Dict[str, Tuple[int, ...]]:
     return shapes
 
 
-def random_weights(config: Dict, seed: int, experts_alike: float = 0.75) -> Dict[str, np.ndarray]:
+def random_weights(config: Dict, seed: int, experts_alike: float = 0.9) -> Dict[str, np.ndarray]:
     """Weights that make every part count: matrices keep the size of what passes through them (the router's and the
     units' somewhat more, so that the clamps bite), decays from barely forgetting to forgetting at once, biases and
     taps of visible size. The experts of a layer share ``experts_alike`` of their weights: where bfloat16 rounding turns

@@ -731,7 +731,7 @@ def test_attention_decode_on_the_matrix_cores(ops, nh, nkv, hd, window):
             ctypes.c_void_p(q.data_ptr()), ctypes.c_void_p(out.data_ptr()), ctypes.c_void_p(partial.data_ptr()), 1, 100000,
             None, None, 0, ctypes.c_void_p(k_pages.data_ptr()), ctypes.c_void_p(v_pages.data_ptr()), ctypes.c_void_p(d(table).data_ptr()),
             table.shape[1], ctypes.c_void_p(d(np.arange(rows)).data_ptr()), ctypes.c_void_p(d(positions).data_ptr()), rows, nh,
-            nkv, hd, hd, ctypes.c_float(scale), 0, 0, ctypes.c_float(0.0), 0, None, 64, 40, None)
+            nkv, hd, hd, ctypes.c_float(scale), 0, 0, ctypes.c_float(0.0), 0, None, None, 64, 40, None)
         ops._check(status)
 
 
