@@ -357,11 +357,12 @@ int fw_causal_conv(const float* in, int in_stride, const float* taps, const floa
 // a = exp(-rate * r * softplus(lam[c])), S <- a S + sqrt(1 - a^2) * i * u[c], out[c] = S * gelu_tanh(y[c]). The gates of a
 // block of block_width channels lie side by side, [r of the block | i of the block], block after block (gates rows of
 // gates_stride >= 2 * channels floats). state float32 [slots][channels], read at a segment's start, written at its end.
-// All float32; out [rows][channels] of out_dtype.
+// All float32; out [rows][channels] of out_dtype. workspace: null, or 2 * rows * channels floats: segments of more than 256
+// rows are then walked in chunks of 64 rows side by side (their sums differ from the walk in order by rounding alone).
 int fw_rglru_scan(const float* u, int u_stride, const float* gates, int gates_stride, const float* y, int y_stride,
                   const float* r_bias, const float* i_bias, const float* lam, float rate, float* state, const int32_t* seg_row0,
                   const int32_t* seg_slot, void* out, int out_dtype, int rows, int segments, int channels, int block_width,
-                  int slots, void* stream);
+                  int slots, float* workspace, void* stream);
 
 #ifdef __cplusplus
 }

@@ -136,6 +136,36 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__
     }
 }
 
+// Few rows of float32 inputs against bfloat16 weights (a decode step's gates of a recurrence, which stay float32): a wave
+// per output, its lanes along k, every row's sum through the wave; the weights are read once, in runs along k. Float32
+// products and sums; a row's sum does not depend on the rows beside it.
+#define HL_FEW_ROWS 16
+template <typename TW>
+__global__ __launch_bounds__(256) void head_linear_few_rows_kernel(const float* __restrict__ in, int in_stride, const TW* __restrict__ w,
+                                                                  float* __restrict__ out, int rows, int heads, int N, int K, int in_head,
+                                                                  int out_head, int out_stride) {
+    const int head = blockIdx.y;
+    const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (n >= N) return;
+    const TW* w_row = w + ((size_t)head * N + n) * K;
+    const float* from = in + (size_t)head * in_head;
+    float acc[HL_FEW_ROWS];
+#pragma unroll
+    for (int r = 0; r < HL_FEW_ROWS; ++r) acc[r] = 0.0f;
+    for (int k = lane; k < K; k += 64) {
+        const float wv = load_as_float(w_row, k);
+#pragma unroll
+        for (int r = 0; r < HL_FEW_ROWS; ++r)
+            if (r < rows) acc[r] = fmaf(from[(size_t)r * in_stride + k], wv, acc[r]);
+    }
+#pragma unroll
+    for (int r = 0; r < HL_FEW_ROWS; ++r) {
+        if (r >= rows) break;
+        const float sum = wave_sum(acc[r]);
+        if (lane == 0) out[(size_t)r * out_stride + (size_t)head * out_head + n] = sum;
+    }
+}
+
 // The same on the matrix cores, bfloat16 in, float32 sums, bfloat16 out. A wave forms 16 rows by 16 NT outputs of
 // one head: per 32 values of k one operand of the rows and NT of the weights, each lane's eight values
 // one 16-byte load straight from memory (K and the rows' stride multiples of 8), no LDS: the weights of a head are
@@ -229,6 +259,12 @@ extern "C" int fw_head_linear(const void* in, int in_dtype, int in_stride, const
             head_linear_mfma_kernel<4, false><<<tall, 256, 0, s>>>((const uint16_t*)in, in_stride, (const uint16_t*)w, gate, gate_stride,
                                                                    (uint16_t*)out, rows, heads, N, K, in_head, out_head, out_stride);
         }
+        FW_LAUNCH_CHECK("head_linear");
+        return 0;
+    }
+    if (rows <= HL_FEW_ROWS && in_dtype == FW_F32 && w_dtype == FW_BF16 && out_dtype == FW_F32 && gate == nullptr) {
+        head_linear_few_rows_kernel<bf16_t><<<dim3((N + 3) / 4, heads), 256, 0, s>>>((const float*)in, in_stride, (const bf16_t*)w, (float*)out, rows,
+                                                                                     heads, N, K, in_head, out_head, out_stride);
         FW_LAUNCH_CHECK("head_linear");
         return 0;
     }

@@ -1583,6 +1583,9 @@ def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor
     return out
 
 
+SCAN_LONG = 256     # rows of a segment beyond which the recurrence walks it in chunks side by side
+
+
 def rglru_scan(u: torch.Tensor, gates: torch.Tensor, y: torch.Tensor, r_bias: torch.Tensor, i_bias: torch.Tensor, lam: torch.Tensor,
                rate: float, state: torch.Tensor, seg_row0: torch.Tensor, seg_slot: torch.Tensor, segments: int, block_width: int,
                out_dtype: torch.dtype) -> torch.Tensor:
@@ -1605,11 +1608,13 @@ def rglru_scan(u: torch.Tensor, gates: torch.Tensor, y: torch.Tensor, r_bias: to
         if t.numel() < n:
             raise KernelError(f"rglru_scan: {name} holds {t.numel()} entries, needs {n}")
     out = torch.empty((rows, channels), dtype=out_dtype, device=u.device)
+    # a step that may hold a long segment: the kernels walk such a one in chunks side by side and need room for it
+    workspace = torch.empty((2, rows, channels), dtype=torch.float32, device=u.device) if rows > SCAN_LONG else None
 
     def stride(t: torch.Tensor) -> int:
         return t.stride(0) if rows > 1 else max(channels, t.stride(0))
 
     _check(library().fw_rglru_scan(_p(u), stride(u), _p(gates), 2 * channels, _p(y), stride(y), _p(r_bias), _p(i_bias), _p(lam),
                                    ctypes.c_float(rate), _p(state), _p(seg_row0), _p(seg_slot), _p(out), _code(out_dtype), rows,
-                                   int(segments), channels, int(block_width), state.shape[0], _stream()))
+                                   int(segments), channels, int(block_width), state.shape[0], _p(workspace), _stream()))
     return out

@@ -83,9 +83,11 @@ def plain_scan(u, gates, y, r_bias, i_bias, lam, S, block):
 
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
-@pytest.mark.parametrize("channels,block,lengths", [(12, 4, [1, 5, 1, 2]), (300, 100, [70, 9]), (64, 64, [1, 1, 1]), (50, 1, [17])])
+@pytest.mark.parametrize("channels,block,lengths", [(12, 4, [1, 5, 1, 2]), (300, 100, [70, 9]), (64, 64, [1, 1, 1]), (50, 1, [17]),
+                                                    (96, 32, [700, 3, 257, 256]), (40, 8, [1000])])
 def test_rglru_scan(ops, channels, block, lengths, out_dtype):
-    """Two steps over the same requests: decays from barely forgetting to forgetting at once, states carried in slots."""
+    """Two steps over the same requests: decays from barely forgetting to forgetting at once, states carried in slots;
+    segments of more than 256 rows are walked in chunks side by side, beside short ones walked in order."""
     rng = np.random.default_rng(channels + block)
     lam, r_bias, i_bias = rng.uniform(-6.0, 1.5, channels), rng.normal(size=channels), rng.normal(size=channels)
     slots = [4, 1, 0, 2][:len(lengths)]
@@ -104,6 +106,19 @@ def test_rglru_scan(ops, channels, block, lengths, out_dtype):
             assert np.abs(found[at:at + n] - want).max() <= limit * max(1.0, np.abs(want).max()), f"step {step} slot {slot}"
             assert np.abs(host(state[slot]) - carried[slot]).max() <= 2e-5 * max(1.0, np.abs(carried[slot]).max())
             at += n
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 17])
+@pytest.mark.parametrize("blocks,width", [(3, 40), (10, 256), (1, 7)])
+def test_the_gates_maps_per_block(ops, rows, blocks, width):
+    """Both gates of a block from one map per block, float32 inputs against bfloat16 weights: few rows (a wave per
+    output) and more (tiles), the same numbers to float32 rounding."""
+    rng = np.random.default_rng(rows + width)
+    u = rng.normal(size=(rows, blocks * width))
+    maps = host(dev(rng.normal(size=(blocks, 2 * width, width)) * width ** -0.5, torch.bfloat16))
+    found = host(ops.head_linear(dev(u), dev(maps, torch.bfloat16), torch.float32))
+    want = np.einsum("bnk,rbk->rbn", maps, host(dev(u)).reshape(rows, blocks, width)).reshape(rows, -1)
+    assert np.abs(found - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
 
 
 def test_rglru_scan_gives_the_same_bits_however_the_tokens_are_cut(ops):
