@@ -140,23 +140,40 @@ __global__ __launch_bounds__(256) void head_linear_kernel(const TI* __restrict__
 // per output, its lanes along k, every row's sum through the wave; the weights are read once, in runs along k. Float32
 // products and sums; a row's sum does not depend on the rows beside it.
 #define HL_FEW_ROWS 16
-template <typename TW>
-__global__ __launch_bounds__(256) void head_linear_few_rows_kernel(const float* __restrict__ in, int in_stride, const TW* __restrict__ w,
+// VEC: K, the rows' stride and the heads' offsets are multiples of 4 and the pointers 16-byte aligned: a lane takes four
+// neighbouring k at a time, the weights' as one 8-byte load and each row's as one of 16 bytes, all asked for together.
+template <bool VEC>
+__global__ __launch_bounds__(256) void head_linear_few_rows_kernel(const float* __restrict__ in, int in_stride, const uint16_t* __restrict__ w,
                                                                   float* __restrict__ out, int rows, int heads, int N, int K, int in_head,
                                                                   int out_head, int out_stride) {
     const int head = blockIdx.y;
     const int n = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (n >= N) return;
-    const TW* w_row = w + ((size_t)head * N + n) * K;
+    const uint16_t* w_row = w + ((size_t)head * N + n) * K;
     const float* from = in + (size_t)head * in_head;
     float acc[HL_FEW_ROWS];
 #pragma unroll
     for (int r = 0; r < HL_FEW_ROWS; ++r) acc[r] = 0.0f;
-    for (int k = lane; k < K; k += 64) {
-        const float wv = load_as_float(w_row, k);
+    if (VEC) {
+        typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+        typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+        for (int k = lane * 4; k < K; k += 256) {
+            const u32x2_t bits = *reinterpret_cast<const u32x2_t*>(w_row + k);
+            f32x4_t x[HL_FEW_ROWS];
 #pragma unroll
-        for (int r = 0; r < HL_FEW_ROWS; ++r)
-            if (r < rows) acc[r] = fmaf(from[(size_t)r * in_stride + k], wv, acc[r]);
+            for (int r = 0; r < HL_FEW_ROWS; ++r) x[r] = *reinterpret_cast<const f32x4_t*>(from + (size_t)(r < rows ? r : rows - 1) * in_stride + k);
+            const float w0 = __uint_as_float(bits[0] << 16), w1 = __uint_as_float(bits[0] & 0xffff0000u);
+            const float w2 = __uint_as_float(bits[1] << 16), w3 = __uint_as_float(bits[1] & 0xffff0000u);
+#pragma unroll
+            for (int r = 0; r < HL_FEW_ROWS; ++r) acc[r] = fmaf(x[r][3], w3, fmaf(x[r][2], w2, fmaf(x[r][1], w1, fmaf(x[r][0], w0, acc[r]))));
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) {
+            const float wv = __uint_as_float((uint32_t)w_row[k] << 16);
+#pragma unroll
+            for (int r = 0; r < HL_FEW_ROWS; ++r)
+                if (r < rows) acc[r] = fmaf(from[(size_t)r * in_stride + k], wv, acc[r]);
+        }
     }
 #pragma unroll
     for (int r = 0; r < HL_FEW_ROWS; ++r) {
@@ -263,8 +280,13 @@ extern "C" int fw_head_linear(const void* in, int in_dtype, int in_stride, const
         return 0;
     }
     if (rows <= HL_FEW_ROWS && in_dtype == FW_F32 && w_dtype == FW_BF16 && out_dtype == FW_F32 && gate == nullptr) {
-        head_linear_few_rows_kernel<bf16_t><<<dim3((N + 3) / 4, heads), 256, 0, s>>>((const float*)in, in_stride, (const bf16_t*)w, (float*)out, rows,
-                                                                                     heads, N, K, in_head, out_head, out_stride);
+        const bool vec = K % 4 == 0 && in_stride % 4 == 0 && in_head % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)w % 8 == 0;
+        if (vec)
+            head_linear_few_rows_kernel<true><<<dim3((N + 3) / 4, heads), 256, 0, s>>>((const float*)in, in_stride, (const uint16_t*)w, (float*)out,
+                                                                                       rows, heads, N, K, in_head, out_head, out_stride);
+        else
+            head_linear_few_rows_kernel<false><<<dim3((N + 3) / 4, heads), 256, 0, s>>>((const float*)in, in_stride, (const uint16_t*)w, (float*)out,
+                                                                                        rows, heads, N, K, in_head, out_head, out_stride);
         FW_LAUNCH_CHECK("head_linear");
         return 0;
     }

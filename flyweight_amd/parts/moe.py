@@ -132,6 +132,7 @@ class MoeSwiGLU(FeedForward):
         return None
 
     def output(self, h, ctx) -> torch.Tensor:
-        out = torch.zeros((h.shape[0], self.hidden), dtype=torch.float32, device=h.device)
+        out = torch.empty((h.shape[0], self.hidden), dtype=torch.float32, device=h.device)
+        ops.fill_zero(out)
         self.forward(h, out, ctx)
         return out
