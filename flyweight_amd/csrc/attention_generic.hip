@@ -10,7 +10,7 @@
 #include "fw_kernels.h"
 
 #define ATTN_PAGE 64
-#define ATTN_MAX_HEAD_DIM 512       // of these plain kernels (the matrix-core kernels take up to 256)
+#define ATTN_MAX_HEAD_DIM 1024      // of these plain kernels (the matrix-core kernels take up to 256)
 
 // One wave per (row, head-vector). Head-vectors 0..nh-1 are queries, nh..nh+nkv-1 keys (head_dim
 // channels each), the rest values (v_dim channels each, which may differ from head_dim). Per-head RMS norm then half-split rotation: channel i pairs with

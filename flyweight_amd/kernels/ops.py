@@ -19,7 +19,7 @@ from . import build as _build
 F32, BF16 = 0, 1
 PAGE_SIZE = 64          # tokens per cache page: the width of a wavefront
 MAX_HEAD_DIM = 256          # of the matrix-core attention kernels
-MAX_PLAIN_HEAD_DIM = 512    # of the plain attention kernels, which serve what the others do not take
+MAX_PLAIN_HEAD_DIM = 1024   # of the plain attention kernels, which serve what the others do not take
 ABI_VERSION = 16
 
 _lib = None

@@ -212,27 +212,6 @@ def route(h: np.ndarray, router: np.ndarray, top: int, groups: int, keep: int) -
     return chosen, weight
 
 
-def route_margin(h: np.ndarray, router: np.ndarray, top: int, groups: int, keep: int) -> np.ndarray:
-    """How clear each row's choice is, [T]: the smallest gap between what is chosen and what is not (the last kept
-    group's best logit against the first group left out, the last chosen expert's logit against the first one left
-    out), as a fraction of the row's largest logit in size. Rows near 0 are close calls: a rounding of h can turn them."""
-    z = h @ router.T
-    T, E = z.shape
-    margin = np.full(T, np.inf)
-    for t in range(T):
-        allowed = z[t].copy()
-        if groups > 1 and keep < groups:
-            best = np.sort(z[t].reshape(groups, E // groups).max(axis=1))[::-1]
-            margin[t] = best[keep - 1] - best[keep]
-            kept = np.argsort(-z[t].reshape(groups, E // groups).max(axis=1), kind="stable")[:keep]
-            allowed = np.concatenate([z[t, g * (E // groups):(g + 1) * (E // groups)] for g in kept])
-        if top < allowed.size:
-            ordered = np.sort(allowed)[::-1]
-            margin[t] = min(margin[t], ordered[top - 1] - ordered[top])
-        margin[t] /= max(np.abs(z[t]).max(), 1e-30)
-    return margin
-
-
 def mixture(h: np.ndarray, w: Dict[str, np.ndarray], sizes: Dict) -> np.ndarray:
     """sizes: experts, top, groups, keep, limit, and shared_limit where there is a shared unit."""
     chosen, weight = route(h, w["router"], sizes["top"], sizes["groups"], sizes["keep"])
@@ -282,9 +261,9 @@ class PlainTelapel:
     def start(self) -> List:
         return [None] * len(self.config["layers"])
 
-    def forward(self, tokens, states: Optional[List] = None, keep_layers: bool = False, margins: Optional[List] = None):
+    def forward(self, tokens, states: Optional[List] = None, keep_layers: bool = False):
         """Logits [T, vocab] of the next ``tokens`` of one sequence; ``states`` (from ``start`` or an earlier
-        call) is brought up to date in place. ``margins``: a list that receives every mixture's ``route_margin``."""
+        call) is brought up to date in place."""
         if states is None:
             states = self.start()
         x = self.tensors["embed"][np.asarray(tokens, dtype=np.int64)]
@@ -301,9 +280,6 @@ class PlainTelapel:
                 y, states[index] = key_value_attention(x, mix, _mixer_sizes(entry), self.eps, states[index])
             x = x + rms_norm(y, w["norm1"], self.eps)
             if entry.get("mlp") is not None:
-                if margins is not None:
-                    sizes = _ff_sizes(entry["mlp"])
-                    margins.append(route_margin(x, w["mlp.router"], sizes["top"], sizes["groups"], sizes["keep"]))
                 x = x + rms_norm(mixture(x, _under(w, "mlp."), _ff_sizes(entry["mlp"])), w["norm2"], self.eps)
             after.append(x.copy())
         logits = rms_norm(x, self.tensors["final.norm"], self.eps) @ self.tensors["embed"].T

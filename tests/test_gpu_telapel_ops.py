@@ -315,7 +315,7 @@ def test_the_term_of_one_and_the_bias_by_distance(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,d,window,softcap", [(6, 2, 32, 50, 20.0), (4, 4, 16, 33, 8.0), (2, 1, 48, 64, 0.0), (3, 1, 20, 0, 50.0), (8, 2, 64, 150, 30.0)])
+@pytest.mark.parametrize("H,G,d,window,softcap", [(6, 2, 32, 50, 20.0), (4, 4, 16, 33, 8.0), (2, 1, 48, 64, 0.0), (3, 1, 20, 0, 50.0), (8, 2, 64, 150, 30.0), (10, 2, 32, 40, 20.0)])
 def test_attention_against_the_plain_heads(ops, dtype, H, G, d, window, softcap):
     """Rows at several positions of a sequence of 200 (in the first window, across page borders, at the end), and in
     bfloat16 the whole sequence as one prompt and as a portion behind cached keys, through the prompt kernel."""
@@ -338,9 +338,13 @@ def test_attention_against_the_plain_heads(ops, dtype, H, G, d, window, softcap)
             seg_row0 = [0, T - first]
             tile_seg, tile_row0 = ops.query_tiles(seg_row0)
             q = dev(q_all[first:].reshape(T - first, H * d), dtype)
-            found = ops.attention_prefill(q, H, G, d, k_pages, v_pages, ints([pages]), ints(tile_seg), ints(tile_row0), ints(seg_row0),
-                                          ints(np.arange(first, T)), scale, window, softcap=softcap, sinks=dev(np.zeros(H)), slopes=dev(slopes_of(H)))
-            assert np.abs(host(found).reshape(-1, H, d) - expected[first:]).max() <= limit * max(1.0, np.abs(expected).max()), f"rows from {first}"
+            # one query head to a workgroup, and four heads of a key head together where the kernel has that form
+            for together in (1, 4) if d <= 64 and H // G >= 4 else (1,):
+                found = ops.attention_prefill(q, H, G, d, k_pages, v_pages, ints([pages]), ints(tile_seg), ints(tile_row0), ints(seg_row0),
+                                              ints(np.arange(first, T)), scale, window, heads_together=together, softcap=softcap,
+                                              sinks=dev(np.zeros(H)), slopes=dev(slopes_of(H)))
+                assert np.abs(host(found).reshape(-1, H, d) - expected[first:]).max() <= limit * max(1.0, np.abs(expected).max()), \
+                    f"rows from {first}, {together} heads together"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
