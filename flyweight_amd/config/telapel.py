@@ -10,9 +10,9 @@ per-head norm, a query factor that grows with the position ``q_temp.coef`` / ``q
 a bias by distance, a sliding window ``mask.size`` and a softmax with one more term of 1 in its denominator, see
 ``parts/attention.py``). ``mlp`` is ``null`` or ``{"kind": "moe", "router": {"experts", "top", "groups": {"count", "keep"}},
 "expert": {"ff", "limit"}, "shared": {"ff", "limit"}}``: a mixture of clamped gated units chosen among the best groups of
-experts, with one unit that every token runs. A layer with ``weights_of: j`` has no tensors of its own: it runs layer j's
-weights on a cache entry or state of its own. The head is the embedding table behind the final norm. A checkpoint names
-its tensors ``l<i>.<part>`` without a ".weight" suffix.
+experts, with one unit that every token runs. An entry with ``weights_of: j`` brings no weights: the layer is run with those
+that layer j loaded, while its pages or its slot are kept apart from layer j's. The head is the embedding table behind the
+final norm. A checkpoint names its tensors ``l<i>.<part>`` without a ".weight" suffix.
 """
 
 from __future__ import annotations
@@ -202,7 +202,7 @@ class TelapelConfig:
                 continue
             where = f"layers[{index}].weights_of"
             if layer.weights_of >= len(layers) or layer.weights_of == index or layers[layer.weights_of].weights_of is not None:
-                raise ConfigError(f"config.json: {where} = {layer.weights_of} must name another layer that has tensors of its own")
+                raise ConfigError(f"config.json: {where} = {layer.weights_of} must name another layer, one that loads weights itself")
             owner = layers[layer.weights_of]
             if (owner.mixer, owner.mlp) != (layer.mixer, layer.mlp):
                 raise ConfigError(f"config.json: {where}: a layer that runs layer {layer.weights_of}'s weights has that layer's sizes")

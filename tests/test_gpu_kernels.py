@@ -389,8 +389,8 @@ def test_kernels_refuse_what_they_were_not_written_for(ops):
     with pytest.raises(KernelError, match="float32 or bfloat16"):
         ops.gemm(x.half(), torch.zeros(4, 8, device=DEV).half())
     with pytest.raises(KernelError, match="head_dim"):
-        ops.attention_generic(torch.zeros(1, 1024, device=DEV), 1, 1, 1024, torch.zeros(1, 1, 64, 1024, device=DEV),
-                              torch.zeros(1, 1, 1024, 64, device=DEV), torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+        ops.attention_generic(torch.zeros(1, 2048, device=DEV), 1, 1, 2048, torch.zeros(1, 1, 64, 2048, device=DEV),
+                              torch.zeros(1, 1, 2048, 64, device=DEV), torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                               torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV), 1.0)
     with pytest.raises(KernelError, match="kernel size"):
         ops.shortconv(torch.zeros(1, 24, device=DEV), torch.zeros(8, 17, device=DEV), None, torch.zeros(1, 8, 16, device=DEV),
