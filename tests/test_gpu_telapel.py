@@ -165,6 +165,19 @@ def test_each_mixer_alone(models, name, variant, dtype):
     assert_close(feed(stepper, "c", tokens, [5, 2, 70, 1, 1]), loaded.expected(tokens), dtype, f"{name} {variant} cut")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_latent_wider_than_the_matrix_core_kernels_take(dtype, tmp_path):
+    """A latent of 512 channels with a rotated part of 64: keys of 576 channels go to the plain attention kernel in
+    both dtypes; whole, cut, and with a decoded tail."""
+    config = model(150, 64, [layer(latent(2, 32, 64, 16, 24, 512, 0.1), None), layer(rglru(32, 2, 3), moe(4, 2, 2, 1, 16, 1.0))])
+    loaded = Loaded(str(tmp_path / dtype), config, dtype, seed=3)
+    tokens = random_tokens(config["vocab"], 100, seed=5)
+    for cuts in ([100], [33, 2, 65], [80] + [1] * 20):
+        stepper = loaded.stepper(num_pages=3, max_requests=2)
+        stepper.admit("a")
+        assert_close(feed(stepper, "a", tokens, cuts), loaded.expected(tokens), dtype, f"wide latent cut {cuts[:3]}")
+
+
 def random_config(seed):
     """Two to six layers of any mixer in any order, every size drawn: heads and groups of 1..4, head sizes on and off
     the matrix cores' steps of 16, windows of 1 token to longer than the prompt or none, with and without a cap and a
